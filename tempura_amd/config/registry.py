@@ -12,6 +12,7 @@ import os
 from typing import Any, Callable, Dict
 
 from .llama import ConfigError, LlamaConfig
+from .mifutar import MifutarConfig
 
 _ARCHITECTURES: Dict[str, Any] = {}
 
@@ -56,10 +57,13 @@ def load_config(model_dir: str):
         name = archs[0]
     elif d.get("model_type") is not None:
         name = d["model_type"]
+    elif d.get("architecture") is not None:
+        name = d["architecture"]
     else:
-        raise ConfigError(f"{path}: neither 'architectures' nor 'model_type' names the model")
+        raise ConfigError(f"{path}: none of 'architectures', 'model_type' and 'architecture' names the model")
     return config_class_for(str(name)).from_dict(d)
 
 
 register_architecture("LlamaForCausalLM", LlamaConfig)
 register_architecture("llama", LlamaConfig)
+register_architecture("Mifutar", MifutarConfig)

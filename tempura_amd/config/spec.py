@@ -85,6 +85,9 @@ class ModelSpec:
     lm_head: PartSpec
     eos_token_ids: List[int] = field(default_factory=list)
     bos_token_id: Optional[int] = None
+    #: copies of the residual stream that the blocks keep side by side (1: the plain residual stream).  The
+    #: embedding's output starts every copy; the final norm reads their sum.
+    streams: int = 1
 
     def resolved_order(self) -> List[LayerCall]:
         """The run order with every call's cache slot made explicit.

@@ -10,6 +10,9 @@
 // Query token t belongs to request r = token_req[t]; its position is
 // context_lens[r] - q_len_r + (t - cu_seqlens[r]) and it sees keys lo..pos with
 // lo = max(0, pos - window + 1) when window > 0, else 0.
+//
+// Optional bias by distance: dist_bias [heads, bias_len] float32 is added to the scaled score of query position
+// pos and key j as dist_bias[h, min(pos - j, bias_len - 1)] (the scale does not multiply it).
 #include <math.h>
 
 #include "common.h"
@@ -21,7 +24,7 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_seqlens,
     const int* __restrict__ context_lens, const int* __restrict__ token_req, T* __restrict__ out, int n_heads,
-    int n_kv, int head_dim, int page_size, float scale, int window) {
+    int n_kv, int head_dim, int page_size, float scale, int window, const float* __restrict__ dist_bias, int bias_len) {
   extern __shared__ float qs[];  // the query row, float32
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = token_req[t];
@@ -54,6 +57,7 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
       float dot = 0.f;
       for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_float(kr[d]), dot);
       s = dot * scale;
+      if (dist_bias != nullptr) s += dist_bias[(size_t)h * bias_len + min(pos - j, bias_len - 1)];
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float alpha = expf(m - m_new);  // first tile: exp(-inf) = 0
@@ -96,7 +100,7 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
                                   int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale,
                                   int window, int max_q_len, int max_ctx, int allow_fast, int num_single,
                                   int num_splits, float* scratch, int portion_splits, int portion_min_steps,
-                                  float* portion_scratch, hipStream_t s) {
+                                  float* portion_scratch, const float* dist_bias, int bias_len, hipStream_t s) {
   // num_single: how many requests bring exactly one token (they go to the split decode kernel,
   // which, with more than one split, needs `scratch` of n_req * n_heads * num_splits * (head_dim + 2)
   // floats).  portion_splits > 1: the keys of every longer request are split over that many blocks,
@@ -109,7 +113,8 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
   TP_REQUIRE(window >= 0, "paged_attention: window must be >= 0");
   TP_REQUIRE(n_heads <= 65535, "paged_attention: too many heads");
   if (n_tokens == 0) return 0;
-  if (dt == TP_BF16 && allow_fast) {
+  TP_REQUIRE(dist_bias == nullptr || bias_len > 0, "paged_attention: empty distance bias table");
+  if (dt == TP_BF16 && allow_fast && dist_bias == nullptr) {
     const int rc = tp_paged_attention_fast(q, k_cache, v_cache, block_tables, table_width, cu_seqlens,
                                            context_lens, out, n_tokens, n_req, n_heads, n_kv, head_dim,
                                            page_size, scale, window, max_q_len, num_single, num_splits, scratch, token_req,
@@ -121,11 +126,11 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
   if (dt == TP_F32)
     hipLaunchKernelGGL(paged_attention_kernel<float>, grid, dim3(64), shmem, s, (const float*)q,
                        (const float*)k_cache, (const float*)v_cache, block_tables, table_width, cu_seqlens,
-                       context_lens, token_req, (float*)out, n_heads, n_kv, head_dim, page_size, scale, window);
+                       context_lens, token_req, (float*)out, n_heads, n_kv, head_dim, page_size, scale, window, dist_bias, bias_len);
   else if (dt == TP_BF16)
     hipLaunchKernelGGL(paged_attention_kernel<bf16_t>, grid, dim3(64), shmem, s, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_seqlens,
-                       context_lens, token_req, (bf16_t*)out, n_heads, n_kv, head_dim, page_size, scale, window);
+                       context_lens, token_req, (bf16_t*)out, n_heads, n_kv, head_dim, page_size, scale, window, dist_bias, bias_len);
   else
     TP_REQUIRE(false, "paged_attention: unknown dtype %d", dt);
   TP_CHECK_LAUNCH("paged_attention");

@@ -32,6 +32,8 @@ class CausalLM:
         self.final_norm = build_part("norm", spec.final_norm, h, dtype, device)
         self.lm_head = part_class("lm_head", spec.lm_head.kind)(spec.lm_head, h, dtype, device, spec.vocab_size)
         self.order = spec.resolved_order()
+        #: copies of the residual stream that the blocks keep side by side; ``h`` is [tokens, streams * hidden]
+        self.streams = int(getattr(spec, "streams", 1) or 1)
         #: None, or a callable (i, h) called before run-order entry i and once after the last with the residual
         #: stream as it stands (eager passes only; see ``Engine.profile``)
         self.observer = None
@@ -128,22 +130,42 @@ class CausalLM:
         Returns float32 logits [len(ctx.logit_rows), vocab]."""
         if hasattr(ctx, "shared"):
             ctx.shared.clear()      # what layers share is computed anew in every pass (also in one that is captured)
-        h = self.embedding.forward(tokens)
+        if self.streams > 1 or getattr(self.embedding, "inv_freq", None) is not None:
+            h = self.embedding.forward(tokens, ctx.positions, self.streams)
+        else:
+            h = self.embedding.forward(tokens)
         m = h.shape[0]
         x = None      # rows handed from one block to the next (a norm carried by the products around it)
         observe = self.observer
         for i, call in enumerate(self.order):
             if observe is not None:
-                observe(i, h)
+                observe(i, self._stream_sum(h))
             layer = self.layers[call.layer]
             if not hasattr(layer, "entry_norm"):
                 layer.forward(h, ctx, caches[i])
                 x = None
                 continue
             after = self.layers[self.order[i + 1].layer] if i + 1 < len(self.order) else None
-            next_norm = after.entry_norm(m) if hasattr(after, "entry_norm") else None
+            # (a block hands rows only to a block of its own kind: the two agree on what is handed over)
+            same = hasattr(after, "entry_norm") and getattr(after, "handoff", None) == getattr(layer, "handoff", None)
+            next_norm = after.entry_norm(m) if same else None
             x = layer.forward(h, ctx, caches[i], x, next_norm)
         if observe is not None:
-            observe(len(self.order), h)
-        x = self.final_norm.forward(h, ctx.logit_rows)
+            observe(len(self.order), self._stream_sum(h))
+        if self.streams > 1:
+            # the final norm reads the sum of the copies, at the wanted rows only
+            norm = self.final_norm
+            if type(norm).__name__ == "RMSNorm":
+                x = ops.stream_step(h, self.streams, norm_weight=norm.weight, eps=norm.eps, out_dtype=self.dtype,
+                                    rows=ctx.logit_rows, write_back=False)
+            else:
+                x = norm.forward(ops.stream_step(h, self.streams, out_dtype=torch.float32, rows=ctx.logit_rows, write_back=False))
+        else:
+            x = self.final_norm.forward(h, ctx.logit_rows)
         return self.lm_head.forward(x)
+
+    def _stream_sum(self, h: torch.Tensor) -> torch.Tensor:
+        """The residual stream as one tensor [tokens, hidden]: the sum of the copies when there are several."""
+        if self.streams == 1:
+            return h
+        return ops.stream_step(h, self.streams, out_dtype=torch.float32, write_back=False)

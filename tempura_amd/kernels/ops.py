@@ -155,16 +155,205 @@ def _i32(t: torch.Tensor, n: int, what: str) -> None:
 
 
 # ---------------------------------------------------------------------------------
-def embed(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """int32 [n] , [vocab, hidden] -> float32 [n, hidden]."""
+def embed(tokens: torch.Tensor, table: torch.Tensor, positions: Optional[torch.Tensor] = None,
+          inv_freq: Optional[torch.Tensor] = None, streams: int = 1) -> torch.Tensor:
+    """int32 [n] , [vocab, hidden] -> float32 [n, hidden]; with ``streams`` > 1, [n, streams * hidden] holding that
+    many copies of each row.  With ``inv_freq`` (float64 [ceil(hidden / 2)]) and ``positions`` (int32 [n]) a
+    sinusoidal position vector is added: element 2i gets sin(p * inv_freq[i]), element 2i + 1 the cosine."""
     if _backend is not None:
-        return _backend.embed(tokens, table)
-    _dev_ok(tokens, table)
+        if inv_freq is None and streams == 1:
+            return _backend.embed(tokens, table)
+        return _backend.embed(tokens, table, positions, inv_freq, streams)
+    _dev_ok(tokens, table, positions, inv_freq)
     n = tokens.numel()
     _i32(tokens, n, "embed tokens")
     _need(table.dim() == 2, "embed: table must be [vocab, hidden]")
-    out = torch.empty((n, table.shape[1]), dtype=torch.float32, device=table.device)
-    _call("tp_embed", _ptr(tokens), _ptr(table), _dt(table), _ptr(out), n, table.shape[1], _stream())
+    hidden = table.shape[1]
+    if inv_freq is None and streams == 1:
+        out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
+        _call("tp_embed", _ptr(tokens), _ptr(table), _dt(table), _ptr(out), n, hidden, _stream())
+        return out
+    _need(streams >= 1, "embed: streams must be positive")
+    if inv_freq is not None:
+        _need(positions is not None, "embed: positions missing")
+        _i32(positions, n, "embed positions") if n else None
+        _need(inv_freq.dtype == torch.float64 and inv_freq.numel() == (hidden + 1) // 2, "embed: inv_freq must be float64 [ceil(hidden / 2)]")
+    out = torch.empty((n, streams * hidden), dtype=torch.float32, device=table.device)
+    _call("tp_embed_pos", _ptr(tokens), _ptr(positions), _ptr(table), _dt(table), _ptr(inv_freq), _ptr(out), n, hidden,
+          int(streams), _stream())
+    return out
+
+
+def stream_step(h: torch.Tensor, streams: int, y: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+                out_coef: Optional[torch.Tensor] = None, in_coef: Optional[torch.Tensor] = None,
+                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, out_dtype: Optional[torch.dtype] = None,
+                rows: Optional[torch.Tensor] = None, write_back: bool = True) -> Optional[torch.Tensor]:
+    """One step of ``streams`` copies of the residual stream, h float32 [n, streams * width], per row:
+    with ``y`` (float32 [n, width], a sublayer's output) every stream b becomes sum_a mix[a, b] h[a] + out_coef[b] * y
+    (``mix`` float32 [streams, streams], None: identity; ``out_coef`` [streams], None: ones), written back into
+    ``h`` when ``write_back``; then, with ``out_dtype``, the result is u = sum_a in_coef[a] h[a] (None: the plain
+    sum), normed with ``norm_weight`` (float32 [width]; u / sqrt(mean(u^2) + eps) * weight) when that is given,
+    as ``out_dtype`` [n or len(rows), width].  ``rows`` (int32) picks the rows."""
+    if _backend is not None:
+        return _backend.stream_step(h, streams, y, mix, out_coef, in_coef, norm_weight, eps, out_dtype, rows, write_back)
+    _dev_ok(h, y, mix, out_coef, in_coef, norm_weight, rows)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and streams >= 1 and h.shape[1] % streams == 0,
+          "stream_step: h must be float32 [n, streams * width]")
+    n, width = h.shape[0], h.shape[1] // streams
+    if y is not None:
+        _need(y.dtype == torch.float32 and tuple(y.shape) == (n, width), "stream_step: y must be float32 [n, width]")
+    for t, size, what in ((mix, streams * streams, "mix"), (out_coef, streams, "out_coef"), (in_coef, streams, "in_coef"),
+                          (norm_weight, width, "norm_weight")):
+        if t is not None:
+            _need(t.dtype == torch.float32 and t.numel() == size, f"stream_step: {what} must be float32 with {size} elements")
+    n_out = n
+    if rows is not None:
+        n_out = rows.numel()
+        _i32(rows, n_out, "stream_step rows") if n_out else None
+        _need(not (write_back and y is not None) or out_dtype is None, "stream_step: a step over chosen rows cannot write all streams back")
+    out = None
+    if out_dtype is not None:
+        out = torch.empty((n_out, width), dtype=out_dtype, device=h.device)
+        if n_out == 0:
+            return out          # (a step in which no row is wanted)
+    else:
+        _need(y is not None and write_back, "stream_step: nothing to do")
+    _call("tp_hc_step", _ptr(h), _ptr(y), _ptr(mix), _ptr(out_coef), _ptr(in_coef), _ptr(norm_weight), ctypes.c_float(eps),
+          _ptr(out), _dtcode(out_dtype) if out_dtype is not None else _F32, _ptr(rows), n_out, int(streams), width,
+          int(bool(write_back) and y is not None), _stream())
+    return out
+
+
+def scale_(x: torch.Tensor, scale: float) -> torch.Tensor:
+    """x *= scale in place (float32)."""
+    if _backend is not None:
+        return _backend.scale_(x, scale)
+    _dev_ok(x)
+    _need(x.dtype == torch.float32, "scale_: needs float32")
+    _call("tp_scale_f32", _ptr(x), ctypes.c_size_t(x.numel()), ctypes.c_float(scale), _stream())
+    return x
+
+
+def gated_act(gu: torch.Tensor, out_dtype: torch.dtype, slope: float = 1.0, limit: float = 0.0, up_offset: float = 0.0) -> torch.Tensor:
+    """[m, 2i] (gate columns then up columns) -> out_dtype [m, i]: g = min(gate, limit), u = clamp(up, -limit, limit)
+    (limit <= 0: none), g * sigmoid(slope * g) * (u + up_offset)."""
+    if _backend is not None:
+        return _backend.gated_act(gu, out_dtype, slope, limit, up_offset)
+    _dev_ok(gu)
+    _need(gu.dim() == 2 and gu.shape[1] % 2 == 0, "gated_act: input must be [m, 2i]")
+    m, i2 = gu.shape
+    out = torch.empty((m, i2 // 2), dtype=out_dtype, device=gu.device)
+    _call("tp_gated_act", _ptr(gu), _dt(gu), _ptr(out), _dtcode(out_dtype), m, i2 // 2, ctypes.c_float(slope),
+          ctypes.c_float(limit), ctypes.c_float(up_offset), _stream())
+    return out
+
+
+def qk_store(rows: torch.Tensor, q_bias: Optional[torch.Tensor], k_bias: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+             num_heads: int, num_kv_heads: int, head_dim: int, k_cache: Optional[torch.Tensor],
+             v_cache: Optional[torch.Tensor], q_dtype: torch.dtype) -> torch.Tensor:
+    """float32 rows [n, (heads + kv_heads) * head_dim] of a projection (no rotation): biases (float32, per column)
+    are added, q is returned as q_dtype [n, heads, head_dim], k goes to the cache rows ``slots`` of ``k_cache`` and,
+    when ``v_cache`` is given (values that are the keys), into the transposed value cache too.  ``slots`` None: the
+    rows hold q only."""
+    if _backend is not None:
+        return _backend.qk_store(rows, q_bias, k_bias, slots, num_heads, num_kv_heads, head_dim, k_cache, v_cache, q_dtype)
+    _dev_ok(rows, q_bias, k_bias, slots, k_cache, v_cache)
+    _need(rows.dtype == torch.float32 and rows.dim() == 2, "qk_store: rows must be float32 [n, width]")
+    n = rows.shape[0]
+    width = (num_heads + (num_kv_heads if slots is not None else 0)) * head_dim
+    _need(rows.shape[1] == width, f"qk_store: row width {rows.shape[1]} != {width}")
+    for b, size in ((q_bias, num_heads * head_dim), (k_bias, num_kv_heads * head_dim)):
+        if b is not None:
+            _need(b.dtype == torch.float32 and b.numel() == size, "qk_store: bias must be float32, one value per column")
+    page_size, cache_dt = 1, _F32
+    if slots is not None:
+        _i32(slots, n, "slots") if n else None
+        _need(k_cache is not None and k_cache.dim() == 4 and k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == head_dim,
+              "qk_store: k cache must be [pages, kv_heads, page_size, head_dim]")
+        page_size, cache_dt = k_cache.shape[2], _dt(k_cache)
+        if v_cache is not None:
+            _need(tuple(v_cache.shape) == (k_cache.shape[0], num_kv_heads, head_dim, page_size) and v_cache.dtype == k_cache.dtype,
+                  "qk_store: v cache must be [pages, kv_heads, head_dim, page_size] of the key cache's type")
+    q = torch.empty((n, num_heads, head_dim), dtype=q_dtype, device=rows.device)
+    _call("tp_qk_store", _ptr(rows), rows.shape[1], _ptr(q_bias), _ptr(k_bias), _ptr(slots), n, num_heads, num_kv_heads, head_dim,
+          _ptr(q), _dtcode(q_dtype), _ptr(k_cache if slots is not None else None), _ptr(v_cache if slots is not None else None),
+          cache_dt, page_size, _stream())
+    return q
+
+
+def causal_conv(proj: torch.Tensor, col0: int, channels: int, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor,
+                cu_seqlens: torch.Tensor, token_req: torch.Tensor, state_slots: torch.Tensor, num_requests: int) -> torch.Tensor:
+    """Causal convolution per channel over each request's run of tokens, then SiLU.  ``proj`` float32 [n, width]
+    holds the inputs at columns col0 .. col0 + channels; ``weight`` [channels, taps] (last column: the current
+    token), ``bias`` [channels]; ``state`` float32 [slots, row] whose rows start with the carried inputs
+    [taps - 1, channels] (oldest first) of the request in that slot: they are read for the first tokens of a run
+    and replaced by the run's last inputs.  Returns float32 [n, channels]."""
+    if _backend is not None:
+        return _backend.causal_conv(proj, col0, channels, weight, bias, state, cu_seqlens, token_req, state_slots, num_requests)
+    _dev_ok(proj, weight, bias, state, cu_seqlens, token_req, state_slots)
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and 0 <= col0 and col0 + channels <= proj.shape[1], "causal_conv: bad rows")
+    _need(weight.dtype == torch.float32 and weight.dim() == 2 and weight.shape[0] == channels, "causal_conv: weight must be float32 [channels, taps]")
+    taps = weight.shape[1]
+    _need(bias.dtype == torch.float32 and bias.numel() == channels, "causal_conv: bias must be float32 [channels]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= (taps - 1) * channels, "causal_conv: state rows too short")
+    n = proj.shape[0]
+    _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
+    _i32(state_slots, num_requests, "state_slots")
+    _i32(token_req, n, "token_req") if n else None
+    out = torch.empty((n, channels), dtype=torch.float32, device=proj.device)
+    _call("tp_causal_conv", _ptr(proj), proj.shape[1], int(col0), _ptr(weight), _ptr(bias), _ptr(state),
+          ctypes.c_size_t(state.shape[1]), _ptr(cu_seqlens), _ptr(token_req), _ptr(state_slots), _ptr(out), n, int(num_requests),
+          channels, taps, _stream())
+    return out
+
+
+def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col0: int, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
+             state: torch.Tensor, state_off: int, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, num_requests: int,
+             num_heads: int, head_dim: int, state_size: int, groups: int) -> torch.Tensor:
+    """The selective recurrence per head over each request's run: with dt = softplus(proj[:, dt_col0 + h] + dt_bias[h])
+    and a = exp(-exp(a_log[h]) * dt):  S <- a S + dt B x^T,  y = S^T C + d_skip[h] x.  ``xbc`` float32 [n, channels]
+    holds x [heads * head_dim] | B [groups * state] | C [groups * state]; the state [heads, state, head_dim] of a
+    request lives at ``state[slot, state_off:]`` (float32), is read at the start of the run and left as the run
+    leaves it.  Returns y float32 [n, heads * head_dim]."""
+    if _backend is not None:
+        return _backend.ssm_scan(xbc, proj, dt_col0, dt_bias, a_log, d_skip, state, state_off, cu_seqlens, state_slots,
+                                 num_requests, num_heads, head_dim, state_size, groups)
+    _dev_ok(xbc, proj, dt_bias, a_log, d_skip, state, cu_seqlens, state_slots)
+    inner = num_heads * head_dim
+    channels = inner + 2 * groups * state_size
+    _need(xbc.dtype == torch.float32 and xbc.dim() == 2 and xbc.shape[1] == channels, f"ssm_scan: xbc must be float32 [n, {channels}]")
+    n = xbc.shape[0]
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.shape[0] == n and 0 <= dt_col0 and dt_col0 + num_heads <= proj.shape[1],
+          "ssm_scan: bad projection rows")
+    for t in (dt_bias, a_log, d_skip):
+        _need(t.dtype == torch.float32 and t.numel() == num_heads, "ssm_scan: per-head constants must be float32 [heads]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= state_off + num_heads * state_size * head_dim,
+          "ssm_scan: state rows too short")
+    _need(num_heads % groups == 0 and state_size <= 1024, "ssm_scan: heads must be a multiple of groups, state size at most 1024")
+    _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
+    _i32(state_slots, num_requests, "state_slots")
+    y = torch.empty((n, inner), dtype=torch.float32, device=xbc.device)
+    _call("tp_ssm_scan", _ptr(xbc), _ptr(proj), proj.shape[1], int(dt_col0), _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(state),
+          ctypes.c_size_t(state.shape[1]), ctypes.c_size_t(state_off), _ptr(cu_seqlens), _ptr(state_slots), _ptr(y),
+          int(num_requests), num_heads, head_dim, state_size, groups, _stream())
+    return y
+
+
+def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_col0: int, weight: torch.Tensor, eps: float, groups: int,
+                     out_dtype: torch.dtype) -> torch.Tensor:
+    """v = y * silu(proj[:, z_col0 + j]), normed in ``groups`` equal parts (each by its own root mean square, eps
+    inside the root), times ``weight``; float32 in, ``out_dtype`` [n, inner] out."""
+    if _backend is not None:
+        return _backend.gated_group_norm(y, proj, z_col0, weight, eps, groups, out_dtype)
+    _dev_ok(y, proj, weight)
+    _need(y.dtype == torch.float32 and y.dim() == 2, "gated_group_norm: y must be float32 [n, inner]")
+    n, inner = y.shape
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.shape[0] == n and 0 <= z_col0 and z_col0 + inner <= proj.shape[1],
+          "gated_group_norm: bad projection rows")
+    _need(weight.dtype == torch.float32 and weight.numel() == inner and groups > 0 and inner % groups == 0, "gated_group_norm: bad weight or groups")
+    out = torch.empty((n, inner), dtype=out_dtype, device=y.device)
+    _call("tp_gated_group_norm", _ptr(y), _ptr(proj), proj.shape[1], int(z_col0), _ptr(weight), ctypes.c_float(eps), _ptr(out),
+          _dtcode(out_dtype), n, inner, int(groups), _stream())
     return out
 
 
@@ -609,10 +798,15 @@ portion_scratch_limit = 256 << 20
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     cu_seqlens: torch.Tensor, context_lens: torch.Tensor, token_req: torch.Tensor,
                     scale: float, window: int, max_q_len: int, max_context_len: int,
-                    num_single: Optional[int] = None) -> torch.Tensor:
+                    num_single: Optional[int] = None, dist_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [n, heads, head_dim] over k [pages, kv_heads, page_size, head_dim] and transposed
-    v [pages, kv_heads, head_dim, page_size] -> [n, heads * head_dim]."""
+    v [pages, kv_heads, head_dim, page_size] -> [n, heads * head_dim].
+    ``dist_bias`` (float32 [heads, L]): added to the scaled score of a query at position p and a key at j as
+    dist_bias[head, min(p - j, L - 1)]."""
     if _backend is not None:
+        if dist_bias is not None:
+            return _backend.paged_attention(q, k_cache, v_cache, block_tables, cu_seqlens, context_lens,
+                                            token_req, scale, window, max_q_len, max_context_len, dist_bias=dist_bias)
         return _backend.paged_attention(q, k_cache, v_cache, block_tables, cu_seqlens, context_lens,
                                         token_req, scale, window, max_q_len, max_context_len)
     # num_single: requests that bring exactly one token (None: all of them iff max_q_len == 1, else unknown
@@ -635,7 +829,12 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     if num_single is None:
         num_single = r if max_q_len == 1 else 0
     _need(0 <= num_single <= r, "paged_attention: num_single out of range")
-    fast = allow_fast_attention and q.dtype == torch.bfloat16 and d % 32 == 0 and d <= 128 and page_size % 8 == 0
+    if dist_bias is not None:
+        _dev_ok(dist_bias)
+        _need(dist_bias.dtype == torch.float32 and dist_bias.dim() == 2 and dist_bias.shape[0] == heads and dist_bias.shape[1] > 0,
+              "paged_attention: dist_bias must be float32 [heads, L]")
+    # (the matrix-core kernels have no distance bias)
+    fast = allow_fast_attention and q.dtype == torch.bfloat16 and d % 32 == 0 and d <= 128 and page_size % 8 == 0 and dist_bias is None
     splits, scratch = 1, None
     if fast and num_single > 0:
         # enough blocks to fill 256 CUs, but at least 128 keys per block
@@ -683,7 +882,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _call("tp_paged_attention", _ptr(q), _dt(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), width,
           _ptr(cu_seqlens), _ptr(context_lens), _ptr(token_req), _ptr(out), n, r, heads, kvh, d, page_size,
           ctypes.c_float(scale), int(window), int(max_q_len), int(max_context_len), int(fast),
-          int(num_single), int(splits), _ptr(scratch), int(parts), max(1, portion_min_keys // 32), _ptr(part_scratch), _stream())
+          int(num_single), int(splits), _ptr(scratch), int(parts), max(1, portion_min_keys // 32), _ptr(part_scratch),
+          _ptr(dist_bias), 0 if dist_bias is None else dist_bias.shape[1], _stream())
     return out
 
 

@@ -8,13 +8,46 @@ output projection added into the residual stream
 /root/reference/kernels/src/attention.rs:28-87).
 A window of ``w`` lets query position p see keys p-w+1 .. p
 (/root/reference/kernels/src/attention.rs:55-59).
+
+Options beyond that, each a parameter of the part:
+* ``bias``: the q and k projections have biases (tensors ``q_bias``, ``k_bias``);
+* ``values: "keys"``: there is no value projection, a head's values are its keys as projected;
+* ``distance_bias``: a learned bias per head and distance is added to the scaled score (the scale does not
+  multiply it).  Kind ``"log_buckets"``: the tensor has B rows of one value per head, and distance n reads row
+  n while n < B // 2, else row min(B - 1, B // 2 + floor(ln(n / (B // 2)) / ln(max_distance / (B // 2)) * (B - B // 2))).
+  B is the tensor's own first dimension.
+The first two need a position encoding that does not rotate (``"none"``).
 """
 from __future__ import annotations
+
+import math
 
 import torch
 
 from ..kernels import ops
 from .base import CacheSpec, Mixer, WeightInfo, build_part, part_class, register_part
+
+
+def log_bucket(n: int, buckets: int, max_distance: int) -> int:
+    """The row of a ``log_buckets`` table that distance ``n`` >= 0 reads: exact below half the table, then
+    logarithmic up to ``max_distance``, then the last row."""
+    half = buckets // 2
+    if n < half:
+        return n
+    if half == 0 or max_distance <= half:
+        return buckets - 1
+    return min(buckets - 1, half + int(math.floor(math.log(n / half) / math.log(max_distance / half) * (buckets - half))))
+
+
+def distance_table(rows: torch.Tensor, max_distance: int, window) -> torch.Tensor:
+    """float32 [heads, L] from a ``log_buckets`` tensor [B, heads]: entry n is the bias of distance n; every
+    distance from L - 1 on has the value of entry L - 1 (the last row, or never occurs under the window)."""
+    buckets = rows.shape[0]
+    length = 1
+    while log_bucket(length - 1, buckets, max_distance) < buckets - 1 and (window is None or length < window):
+        length += 1
+    index = torch.tensor([log_bucket(n, buckets, max_distance) for n in range(length)], dtype=torch.long)
+    return rows.to(torch.float32)[index].t().contiguous()
 
 
 class PagedAttention(Mixer):
@@ -23,6 +56,7 @@ class PagedAttention(Mixer):
     #: starts at a multiple of eight positions (and of eight rows of the batch) has its values stored piece by piece
     preferred_portion_align = 8
     split_norm = True      # takes rows whose norm its first product finishes; prepares the next norm in its last
+    returns_output = True  # with ``residual`` None the output comes back instead of being added
 
     def __init__(self, spec, hidden_size, dtype, device):
         super().__init__(spec, hidden_size, dtype, device)
@@ -37,8 +71,24 @@ class PagedAttention(Mixer):
         self.q_dim = self.num_heads * self.head_dim
         self.kv_dim = self.num_kv_heads * self.head_dim
         self.position = build_part("position", p["position"], hidden_size, dtype, device)
+        self.has_bias = bool(p.get("bias", False))
+        values = p.get("values", "own")
+        if values not in ("own", "keys"):
+            raise ValueError(f"attention: values {values!r} unknown (known: own, keys)")
+        self.values_are_keys = values == "keys"
+        self.distance_bias = p.get("distance_bias")
+        if self.distance_bias is not None and self.distance_bias.get("kind") != "log_buckets":
+            raise ValueError(f"attention: distance bias {self.distance_bias.get('kind')!r} unknown (known: log_buckets)")
+        if (self.has_bias or self.values_are_keys) and self.position.rotary() is not None:
+            raise ValueError("attention: projection biases and values that are the keys need a position encoding that does not rotate")
+        if self.has_bias and not self.values_are_keys:
+            raise ValueError("attention: projection biases are supported together with values that are the keys")
+        #: q and k come straight from the projection (biases added, keys stored as keys and as values): no rotation kernel
+        self.plain_qk = self.values_are_keys
+        self.split_norm = not self.plain_qk      # (the plain projection takes finished rows only)
         self.wqkv = None
         self.wo = None
+        self.q_bias = self.k_bias = self.dist_table = None
 
     @classmethod
     def expected_weights(cls, spec, hidden_size):
@@ -48,9 +98,16 @@ class PagedAttention(Mixer):
         out = {
             w["q"]: WeightInfo((q_dim, hidden_size)),
             w["k"]: WeightInfo((kv_dim, hidden_size)),
-            w["v"]: WeightInfo((kv_dim, hidden_size)),
             w["o"]: WeightInfo((hidden_size, q_dim)),
         }
+        if p.get("values", "own") != "keys":
+            out[w["v"]] = WeightInfo((kv_dim, hidden_size))
+        if p.get("bias", False):
+            out[w["q_bias"]] = WeightInfo((q_dim,))
+            out[w["k_bias"]] = WeightInfo((kv_dim,))
+        if p.get("distance_bias") is not None:
+            # (the number of rows is the tensor's own; a configuration may name it for random weights)
+            out[w["distance_bias"]] = WeightInfo((p["distance_bias"].get("buckets"), p["num_heads"]))
         # a position encoding may have tensors of its own (a rotary one has none)
         out.update(part_class("position", p["position"].kind).expected_weights(p["position"], hidden_size))
         return out
@@ -73,8 +130,16 @@ class PagedAttention(Mixer):
 
     def load_weights(self, get):
         w = self.spec.weights
+        if self.has_bias:
+            self.q_bias = self._to_device(get(w["q_bias"]), torch.float32)
+            self.k_bias = self._to_device(get(w["k_bias"]), torch.float32)
+        if self.distance_bias is not None:
+            self.dist_table = self._to_device(distance_table(get(w["distance_bias"]), int(self.distance_bias["max_distance"]),
+                                                             self.window), torch.float32)
         # One [q_dim + 2 kv_dim, hidden] matrix: one product instead of three.
-        parts = [self._paired(get(w["q"])), self._paired(get(w["k"])), get(w["v"])]
+        parts = [self._paired(get(w["q"])), self._paired(get(w["k"]))]
+        if not self.values_are_keys:
+            parts.append(get(w["v"]))
         # (stored tiled where the sizes allow: the products then read whole cache lines)
         self.wqkv = ops.tile_weight(torch.cat([self._to_device(t) for t in parts], dim=0).contiguous())
         self.wo = ops.tile_weight(self._to_device(get(w["o"])))
@@ -87,7 +152,9 @@ class PagedAttention(Mixer):
     def forward(self, x, ctx, cache, residual, next_norm=None):
         rot = self.position.rotary()
         q = None
-        if rot is not None and cache.writes:
+        if self.plain_qk:
+            q = self._project_plain(x, ctx, cache)
+        elif rot is not None and cache.writes:
             rows = x.x if isinstance(x, ops.Prenormed) else x
             if ops.linear_rope_ok(x.shape[0], self.wqkv.shape[0], x.shape[1], self.head_dim, rot[1], cache.k.shape[2],
                                   rows.dtype, cache.k.dtype, isinstance(x, ops.Prenormed)):
@@ -97,14 +164,34 @@ class PagedAttention(Mixer):
                                        self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v, table)
         if q is None:
             q = self._project_and_rotate(x, ctx, cache, rot)
-        a = ops.paged_attention(
-            q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
-            ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,
-            ctx.num_single)
+        if self.dist_table is not None:
+            a = ops.paged_attention(
+                q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
+                ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,
+                ctx.num_single, dist_bias=self.dist_table)
+        else:
+            a = ops.paged_attention(
+                q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
+                ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,
+                ctx.num_single)
+        if residual is None:
+            return ops.linear(a, self.wo, torch.float32)
         if next_norm is None:
             ops.linear(a, self.wo, torch.float32, residual=residual)
             return None
         return ops.linear(a, self.wo, torch.float32, residual=residual, next_norm=next_norm)[1]
+
+    def _project_plain(self, x, ctx, cache):
+        """q ([n, heads, head_dim]) of a projection without rotation: biases added, k stored as keys and, when the
+        values are the keys, as values too (the value cache is transposed, so it is a second store, not a view)."""
+        if isinstance(x, ops.Prenormed):
+            raise ValueError("attention: rows with an unfinished norm need a rotary projection")
+        if cache.writes:
+            rows = ops.linear(x, self.wqkv, torch.float32)
+            return ops.qk_store(rows, self.q_bias, self.k_bias, ctx.slot_mapping[cache.group], self.num_heads,
+                                self.num_kv_heads, self.head_dim, cache.k, cache.v, self.dtype)
+        rows = ops.linear(x, ops.weight_rows(self.wqkv, 0, self.q_dim), torch.float32)
+        return ops.qk_store(rows, self.q_bias, None, None, self.num_heads, self.num_kv_heads, self.head_dim, None, None, self.dtype)
 
     def _project_and_rotate(self, x, ctx, cache, rot):
         """q (rotated, [n, heads, head_dim]) of the projection; k and v go to the cache."""

@@ -12,7 +12,10 @@ product, the part after it finishes them in its first.  The block arranges that 
 """
 from __future__ import annotations
 
-from .base import build_part, part_class, register_part
+import torch
+
+from ..kernels import ops
+from .base import Part, WeightInfo, build_part, part_class, register_part
 
 
 class ArrangedBlock:
@@ -23,19 +26,24 @@ class ArrangedBlock:
 
     category = "block"
     ROLES: dict = {}
+    #: roles a layer may leave out (the attribute is then None)
+    OPTIONAL: frozenset = frozenset()
+    #: what this arrangement hands to the block behind it (blocks of the same kind only): see ``entry_norm``
+    handoff = None
 
     def __init__(self, layer_spec, hidden_size, dtype, device):
         self.layer_spec = layer_spec
-        missing = [name for name in self.ROLES if name not in layer_spec.parts]
+        missing = [name for name in self.ROLES if name not in layer_spec.parts and name not in self.OPTIONAL]
         extra = [name for name in layer_spec.parts if name not in self.ROLES]
         if missing or extra:
             raise ValueError(f"block {layer_spec.block!r} arranges the parts {sorted(self.ROLES)}: "
                              f"missing {missing}, not its own {extra}")
         for name, cat in self.ROLES.items():
-            setattr(self, name, build_part(cat, layer_spec.parts[name], hidden_size, dtype, device))
+            ps = layer_spec.parts.get(name)
+            setattr(self, name, None if ps is None else build_part(cat, ps, hidden_size, dtype, device))
 
     def parts(self):
-        return [getattr(self, name) for name in self.ROLES]
+        return [getattr(self, name) for name in self.ROLES if getattr(self, name) is not None]
 
     def cache_owner(self):
         """The part whose ``cache_spec()`` / ``state_spec()`` this layer's cache slot serves."""
@@ -45,7 +53,9 @@ class ArrangedBlock:
     def expected_weights(cls, layer_spec, hidden_size):
         out = {}
         for name, cat in cls.ROLES.items():
-            ps = layer_spec.parts[name]
+            ps = layer_spec.parts.get(name)
+            if ps is None:
+                continue
             out.update(part_class(cat, ps.kind).expected_weights(ps, hidden_size))
         return out
 
@@ -56,6 +66,7 @@ class ArrangedBlock:
 
 class PreNormBlock(ArrangedBlock):
     ROLES = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "ffn": "ffn"}
+    handoff = "split_norm"
 
     def entry_norm(self, m):
         """What the part before this block needs to prepare this block's first norm for ``m`` rows, or None."""
@@ -85,3 +96,118 @@ class PreNormBlock(ArrangedBlock):
 
 
 register_part("block", "prenorm", PreNormBlock)
+
+
+class HyperConnection(Part):
+    """How a sublayer is wired to ``streams`` copies of the residual stream: its input is
+    sum_a in[a] x_a, and its output y updates every copy at once, x_b <- sum_a mix[a, b] x_a + out[b] * y
+    (``mix`` is indexed [from, to]).  Three small tensors, kept in float32."""
+
+    category = "connection"
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        self.streams = int(spec.params["streams"])
+        self.in_coef = self.out_coef = self.mix = None
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        s, w = int(spec.params["streams"]), spec.weights
+        return {w["in"]: WeightInfo((s,)), w["out"]: WeightInfo((s,)), w["mix"]: WeightInfo((s, s))}
+
+    def load_weights(self, get):
+        w = self.spec.weights
+        self.in_coef = self._to_device(get(w["in"]), torch.float32)
+        self.out_coef = self._to_device(get(w["out"]), torch.float32)
+        self.mix = self._to_device(get(w["mix"]), torch.float32)
+
+
+register_part("connection", "hyper_connection", HyperConnection)
+
+
+class StreamOpening:
+    """What the kernel that closes one sublayer needs to open the next: the input coefficients of its connection
+    (None: the plain sum) and the weight and eps of its norm."""
+    __slots__ = ("in_coef", "weight", "eps")
+
+    def __init__(self, in_coef, weight, eps):
+        self.in_coef, self.weight, self.eps = in_coef, weight, eps
+
+
+class HyperBlock(ArrangedBlock):
+    """Pre-norm sublayers around several copies of the residual stream.  ``h`` is float32 [tokens, streams * hidden].
+    For the mixer and then the feed-forward (which a layer may leave out): u = sum_a in[a] x_a, y = sublayer(norm(u)),
+    then every copy is updated from the old ones (see ``HyperConnection``).  A sublayer without a connection part
+    has the plain residual sum (one copy, x <- x + y).
+
+    One kernel closes a sublayer and opens the next (update of the copies, the next input combination and its
+    norm), also across layers: ``entry_norm`` says what the block before needs for that."""
+    ROLES = {"mixer_norm": "norm", "mixer": "mixer", "mixer_link": "connection",
+             "ffn_norm": "norm", "ffn": "ffn", "ffn_link": "connection"}
+    OPTIONAL = frozenset({"mixer_link", "ffn_norm", "ffn", "ffn_link"})
+    handoff = "streams"
+
+    def __init__(self, layer_spec, hidden_size, dtype, device):
+        super().__init__(layer_spec, hidden_size, dtype, device)
+        if (self.ffn is None) != (self.ffn_norm is None):
+            raise ValueError("block 'hyper': a feed-forward and its norm come together")
+        links = [l for l in (self.mixer_link, self.ffn_link) if l is not None]
+        self.streams = links[0].streams if links else 1
+        if any(l.streams != self.streams for l in links) or (self.streams > 1 and (self.mixer_link is None or (self.ffn is not None and self.ffn_link is None))):
+            raise ValueError("block 'hyper': every sublayer of a layer is wired to the same number of copies")
+        self.hidden_size = hidden_size
+        self.dtype = dtype
+
+    @staticmethod
+    def _opening(norm, link):
+        if hasattr(norm, "weight") and hasattr(norm, "eps") and type(norm).__name__ == "RMSNorm":
+            return StreamOpening(None if link is None else link.in_coef, norm.weight, norm.eps)
+        return None
+
+    def entry_norm(self, m):
+        """What the block before needs to prepare this block's first sublayer input (None: this block does it)."""
+        return self._opening(self.mixer_norm, self.mixer_link)
+
+    def _open(self, h, norm, link):
+        """The normed input of a sublayer from the copies as they stand."""
+        op = self._opening(norm, link)
+        if op is not None:
+            return ops.stream_step(h, self.streams, in_coef=op.in_coef, norm_weight=op.weight, eps=op.eps, out_dtype=self.dtype)
+        u = ops.stream_step(h, self.streams, in_coef=None if link is None else link.in_coef, out_dtype=torch.float32)
+        return norm.forward(u)
+
+    def _close(self, h, y, link, opening):
+        """Update the copies with a sublayer's output; with ``opening`` also return the next sublayer's input."""
+        mix = None if link is None else link.mix
+        out = None if link is None else link.out_coef
+        if opening is None:
+            ops.stream_step(h, self.streams, y, mix, out)
+            return None
+        return ops.stream_step(h, self.streams, y, mix, out, opening.in_coef, opening.weight, opening.eps, self.dtype)
+
+    def _run(self, part, x, ctx, cache, n, device):
+        """A sublayer's output as a tensor of its own, float32 [tokens, hidden]."""
+        args = (x, ctx, cache) if cache is not None else (x, ctx)
+        if getattr(part, "returns_output", False):
+            return part.forward(*args, None)
+        y = torch.zeros((n, self.hidden_size), dtype=torch.float32, device=device)
+        part.forward(*args, y)
+        return y
+
+    def forward(self, h, ctx, cache, x=None, next_norm=None):
+        n = h.shape[0]
+        if x is None:
+            x = self._open(h, self.mixer_norm, self.mixer_link)
+        y = self._run(self.mixer, x, ctx, cache, n, h.device)
+        after = next_norm if isinstance(next_norm, StreamOpening) else None
+        if self.ffn is None:
+            return self._close(h, y, self.mixer_link, after)
+        mid = self._opening(self.ffn_norm, self.ffn_link)
+        x2 = self._close(h, y, self.mixer_link, mid)
+        if x2 is None:
+            x2 = self._open(h, self.ffn_norm, self.ffn_link)
+        y2 = self._run(self.ffn, x2, ctx, None, n, h.device)
+        return self._close(h, y2, self.ffn_link, after)
+
+
+register_part("block", "hyper", HyperBlock)

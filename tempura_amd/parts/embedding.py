@@ -5,6 +5,10 @@
 ``norm(hidden)[rows] @ lm_head^T`` in float32, and when the checkpoint has no
 output matrix the embedding matrix is used for it
 (/root/reference/engine/src/weights.rs:156-166).
+
+Two options beyond that: the embedding may add a sinusoidal position vector (``position: "sinusoid"`` with
+``position_base`` b: element 2i of position p gets sin(p * b^(-2i / hidden)), element 2i + 1 the cosine), and the
+head may multiply its logits by a constant (``scale``).
 """
 from __future__ import annotations
 
@@ -21,6 +25,15 @@ class TokenEmbedding(Part):
         super().__init__(spec, hidden_size, dtype, device)
         self.vocab_size = vocab_size
         self.weight = None
+        kind = spec.params.get("position")
+        if kind not in (None, "sinusoid"):
+            raise ValueError(f"embedding: position {kind!r} unknown (known: sinusoid)")
+        self.inv_freq = None
+        if kind == "sinusoid":
+            base = float(spec.params.get("position_base", 10000.0))
+            i = torch.arange((hidden_size + 1) // 2, dtype=torch.float64)
+            # float64 on the host; the kernel forms the angle in float64 too
+            self.inv_freq = torch.pow(torch.tensor(base, dtype=torch.float64), -2.0 * i / hidden_size).to(device)
 
     @classmethod
     def expected_weights(cls, spec, hidden_size, vocab_size):
@@ -29,9 +42,11 @@ class TokenEmbedding(Part):
     def load_weights(self, get):
         self.weight = self._to_device(get(self.spec.weights["weight"]))
 
-    def forward(self, tokens):
-        """int32 [tokens] -> float32 [tokens, hidden] (the residual stream)."""
-        return ops.embed(tokens, self.weight)
+    def forward(self, tokens, positions=None, streams: int = 1):
+        """int32 [tokens] -> float32 [tokens, streams * hidden]: ``streams`` copies of the residual stream."""
+        if self.inv_freq is None and streams == 1:
+            return ops.embed(tokens, self.weight)
+        return ops.embed(tokens, self.weight, positions, self.inv_freq, streams)
 
 
 class OutputHead(Part):
@@ -42,6 +57,7 @@ class OutputHead(Part):
         self.vocab_size = vocab_size
         self.weight = None
         self.tied = bool(spec.params.get("tied", False))
+        self.scale = float(spec.params.get("scale", 1.0))
 
     @classmethod
     def expected_weights(cls, spec, hidden_size, vocab_size):
@@ -65,7 +81,8 @@ class OutputHead(Part):
 
     def forward(self, x):
         """normed rows [m, hidden] -> float32 logits [m, vocab]."""
-        return ops.linear(x, self.weight, torch.float32)
+        logits = ops.linear(x, self.weight, torch.float32)
+        return logits if self.scale == 1.0 else ops.scale_(logits, self.scale)
 
 
 register_part("embedding", "embedding", TokenEmbedding)

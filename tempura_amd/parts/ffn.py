@@ -54,4 +54,46 @@ class SwiGLU(FeedForward):
         return ops.linear(a, self.w2, torch.float32, residual=residual, next_norm=next_norm)[1]
 
 
+class GatedFFN(FeedForward):
+    """``down(act(gate(x), up(x)))`` with ``act(g, u) = g' * sigmoid(slope * g') * (u' + up_offset)``, where
+    g' = min(g, limit) and u' = clamp(u, -limit, limit) when ``limit`` is given.  slope 1, no limit and offset 0 is
+    SwiGLU; the constants are parameters of the part.  The activation reads the float32 sums of the gate/up
+    product, whatever the compute dtype."""
+    graph_safe = True
+    returns_output = True      # with ``residual`` None the output comes back instead of being added
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        p = spec.params
+        self.intermediate_size = int(p["intermediate_size"])
+        self.slope = float(p.get("sigmoid_slope", 1.0))
+        self.limit = float(p["limit"]) if p.get("limit") is not None else 0.0
+        self.up_offset = float(p.get("up_offset", 0.0))
+        if self.limit < 0:
+            raise ValueError("gated feed-forward: limit must be positive when given")
+        self.w13 = None
+        self.w2 = None
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        i, w = spec.params["intermediate_size"], spec.weights
+        return {
+            w["gate"]: WeightInfo((i, hidden_size)),
+            w["up"]: WeightInfo((i, hidden_size)),
+            w["down"]: WeightInfo((hidden_size, i)),
+        }
+
+    def load_weights(self, get):
+        w = self.spec.weights
+        gate, up = self._to_device(get(w["gate"])), self._to_device(get(w["up"]))
+        self.w13 = ops.tile_weight(torch.cat([gate, up], dim=0).contiguous())      # one product: gate columns, then up
+        self.w2 = ops.tile_weight(self._to_device(get(w["down"])))
+
+    def forward(self, x, ctx, residual=None):
+        gu = ops.linear(x, self.w13, torch.float32)
+        a = ops.gated_act(gu, self.dtype, self.slope, self.limit, self.up_offset)
+        return ops.linear(a, self.w2, torch.float32, residual=residual)
+
+
 register_part("ffn", "swiglu", SwiGLU)
+register_part("ffn", "gated", GatedFFN)

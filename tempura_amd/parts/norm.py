@@ -1,4 +1,7 @@
-"""RMSNorm: ``y = x / sqrt(mean(x^2) + eps) * w``.
+"""RMSNorm: ``y = x / sqrt(mean(x^2) + eps) * (w + weight_offset)``.
+
+``weight_offset`` (default 0) serves checkpoints that store the weight around zero: with 1.0 the stored tensor is
+the deviation from one.  The offset is added once, in float32, when the weight is loaded.
 
 The reference multiplies ``x * scale * w`` with eps inside the square root,
 added to the mean (/root/reference/kernels/src/ggml/ops_llama.rs:201-216).
@@ -18,15 +21,20 @@ class RMSNorm(Norm):
     def __init__(self, spec, hidden_size, dtype, device):
         super().__init__(spec, hidden_size, dtype, device)
         self.eps = float(spec.params["eps"])
+        self.weight_offset = float(spec.params.get("weight_offset", 0.0))
         self.weight = None
 
     @classmethod
     def expected_weights(cls, spec, hidden_size):
-        return {spec.weights["weight"]: WeightInfo((hidden_size,), "ones")}
+        # (a weight stored around zero is drawn like any other tensor, one stored around one as ones)
+        init = "normal" if float(spec.params.get("weight_offset", 0.0)) != 0.0 else "ones"
+        return {spec.weights["weight"]: WeightInfo((hidden_size,), init)}
 
     def load_weights(self, get):
         # Norm weights are tiny and multiply in float32: keep them in float32.
         self.weight = self._to_device(get(self.spec.weights["weight"]), torch.float32)
+        if self.weight_offset != 0.0:
+            self.weight = (self.weight.double() + self.weight_offset).to(torch.float32)
 
     def forward(self, h, rows=None):
         return ops.rmsnorm(h, self.weight, self.eps, self.dtype, rows)

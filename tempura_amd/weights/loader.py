@@ -117,8 +117,11 @@ def check_checkpoint(ckpt: Checkpoint, expected: Dict[str, WeightInfo]) -> None:
     for n, info in expected.items():
         if n not in have:
             continue
-        if tuple(ckpt.shape(n)) != tuple(info.shape):
-            wrong[n] = (tuple(info.shape), tuple(ckpt.shape(n)))
+        # (None in an expected shape: that size is the tensor's own to say)
+        found = tuple(ckpt.shape(n))
+        if len(found) != len(info.shape) or any(e is not None and int(e) != f for e, f in zip(info.shape, found)) or \
+                any(e is None and f < 1 for e, f in zip(info.shape, found)):
+            wrong[n] = (tuple(info.shape), found)
         accepted = ACCEPTED_TAGS[getattr(info, "kind", "float")]
         if ckpt.dtype_tag(n) not in accepted:
             wrong_dt[n] = (accepted, ckpt.dtype_tag(n))

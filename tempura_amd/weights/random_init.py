@@ -52,6 +52,9 @@ def random_tensor(name: str, info: WeightInfo, seed: int, std: float, norm_jitte
     that is float32 or bfloat16 (float16: drawn as float32, then rounded); norm weights are float32 values
     1 + jitter, then converted."""
     key = _tensor_seed(seed, name)
+    if any(d is None for d in info.shape):
+        raise ValueError(f"tensor {name}: the configuration leaves a size to the checkpoint ({tuple(info.shape)}); "
+                         "random weights need it named")
     if info.init == "ones":
         t = torch.ones(info.shape, dtype=torch.float32)
         if norm_jitter:

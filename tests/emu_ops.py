@@ -11,8 +11,108 @@ import torch
 
 
 class EmuOps:
-    def embed(self, tokens, table):
-        return table[tokens.long()].to(torch.float32)
+    def embed(self, tokens, table, positions=None, inv_freq=None, streams=1):
+        x = table[tokens.long()].double()
+        if inv_freq is not None:
+            ang = positions.double()[:, None] * inv_freq.double()[None, :]
+            pe = torch.stack([torch.sin(ang), torch.cos(ang)], dim=2).reshape(x.shape[0], -1)[:, : x.shape[1]]
+            x = x + pe
+        return x.to(torch.float32).repeat(1, streams)
+
+    def stream_step(self, h, streams, y=None, mix=None, out_coef=None, in_coef=None, norm_weight=None, eps=0.0,
+                    out_dtype=None, rows=None, write_back=True):
+        n, width = h.shape[0], h.shape[1] // streams
+        hs = h.double().reshape(n, streams, width)
+        if y is not None:
+            m = torch.eye(streams, dtype=torch.float64) if mix is None else mix.double().reshape(streams, streams)
+            o = torch.ones(streams, dtype=torch.float64) if out_coef is None else out_coef.double()
+            hs = torch.einsum("ab,naw->nbw", m, hs) + o[None, :, None] * y.double()[:, None, :]
+            if write_back:
+                h.copy_(hs.reshape(n, -1).to(torch.float32))
+                hs = h.double().reshape(n, streams, width)
+        if out_dtype is None:
+            return None
+        c = torch.ones(streams, dtype=torch.float64) if in_coef is None else in_coef.double()
+        u = torch.einsum("a,naw->nw", c, hs)
+        if rows is not None:
+            u = u[rows.long()]
+        if norm_weight is not None:
+            u = u / torch.sqrt((u * u).mean(dim=-1, keepdim=True) + eps) * norm_weight.double()
+        return u.to(out_dtype)
+
+    def scale_(self, x, scale):
+        x.mul_(scale)
+        return x
+
+    def gated_act(self, gu, out_dtype, slope=1.0, limit=0.0, up_offset=0.0):
+        i = gu.shape[1] // 2
+        g, u = gu.double()[:, :i], gu.double()[:, i:]
+        if limit > 0:
+            g = torch.clamp(g, max=limit)
+            u = torch.clamp(u, -limit, limit)
+        return (g * torch.sigmoid(slope * g) * (u + up_offset)).to(out_dtype)
+
+    def qk_store(self, rows, q_bias, k_bias, slots, num_heads, num_kv_heads, head_dim, k_cache, v_cache, q_dtype):
+        n = rows.shape[0]
+        q_dim = num_heads * head_dim
+        q = rows.double()[:, :q_dim]
+        if q_bias is not None:
+            q = q + q_bias.double()
+        if slots is not None:
+            k = rows.double()[:, q_dim:]
+            if k_bias is not None:
+                k = k + k_bias.double()
+            k = k.reshape(n, num_kv_heads, head_dim)
+            ps = k_cache.shape[2]
+            page, off = slots.long() // ps, slots.long() % ps
+            k_cache[page, :, off] = k.to(k_cache.dtype)
+            if v_cache is not None:
+                v_cache[page, :, :, off] = k.to(v_cache.dtype)
+        return q.reshape(n, num_heads, head_dim).to(q_dtype).contiguous()
+
+    def causal_conv(self, proj, col0, channels, weight, bias, state, cu_seqlens, token_req, state_slots, num_requests):
+        taps = weight.shape[1]
+        out = torch.zeros(proj.shape[0], channels, dtype=torch.float64)
+        cu = cu_seqlens.tolist()
+        for r in range(num_requests):
+            a, b = cu[r], cu[r + 1]
+            if b <= a:
+                continue
+            slot = int(state_slots[r])
+            carried = state[slot, : (taps - 1) * channels].double().reshape(taps - 1, channels)
+            seq = torch.cat([carried, proj[a:b, col0: col0 + channels].double()], dim=0)
+            for t in range(b - a):
+                out[a + t] = (seq[t: t + taps] * weight.double().T).sum(0) + bias.double()
+            state[slot, : (taps - 1) * channels] = seq[seq.shape[0] - (taps - 1):].reshape(-1).to(torch.float32)
+        return (out * torch.sigmoid(out)).to(torch.float32)
+
+    def ssm_scan(self, xbc, proj, dt_col0, dt_bias, a_log, d_skip, state, state_off, cu_seqlens, state_slots, num_requests,
+                 num_heads, head_dim, state_size, groups):
+        n = xbc.shape[0]
+        H, P, N, G = num_heads, head_dim, state_size, groups
+        inner = H * P
+        x = xbc.double()[:, :inner].reshape(n, H, P)
+        Bm = xbc.double()[:, inner: inner + G * N].reshape(n, G, N).repeat_interleave(H // G, dim=1)
+        Cm = xbc.double()[:, inner + G * N:].reshape(n, G, N).repeat_interleave(H // G, dim=1)
+        dt = torch.nn.functional.softplus(proj.double()[:, dt_col0: dt_col0 + H] + dt_bias.double())
+        decay = torch.exp(-torch.exp(a_log.double()) * dt)
+        y = torch.zeros(n, H, P, dtype=torch.float64)
+        cu = cu_seqlens.tolist()
+        for r in range(num_requests):
+            slot = int(state_slots[r])
+            S = state[slot, state_off: state_off + H * N * P].double().reshape(H, N, P)
+            for t in range(cu[r], cu[r + 1]):
+                S = decay[t, :, None, None] * S + dt[t, :, None, None] * Bm[t, :, :, None] * x[t, :, None, :]
+                y[t] = torch.einsum("hnp,hn->hp", S, Cm[t]) + d_skip.double()[:, None] * x[t]
+            state[slot, state_off: state_off + H * N * P] = S.reshape(-1).to(torch.float32)
+        return y.reshape(n, inner).to(torch.float32)
+
+    def gated_group_norm(self, y, proj, z_col0, weight, eps, groups, out_dtype):
+        n, inner = y.shape
+        z = proj.double()[:, z_col0: z_col0 + inner]
+        v = (y.double() * z * torch.sigmoid(z)).reshape(n, groups, inner // groups)
+        v = v / torch.sqrt((v * v).mean(dim=-1, keepdim=True) + eps)
+        return (v.reshape(n, inner) * weight.double()).to(out_dtype)
 
     def rmsnorm(self, h, weight, eps, out_dtype, rows=None):
         x = h.double()
@@ -93,7 +193,7 @@ class EmuOps:
         return q
 
     def paged_attention(self, q, k_cache, v_cache, block_tables, cu_seqlens, context_lens, token_req, scale,
-                        window, max_q_len, max_context_len, num_single=None):
+                        window, max_q_len, max_context_len, num_single=None, dist_bias=None):
         n, heads, d = q.shape
         kvh, ps = k_cache.shape[1], k_cache.shape[2]
         group = heads // kvh
@@ -112,6 +212,9 @@ class EmuOps:
                 lo = max(0, pos - window + 1) if window > 0 else 0
                 for h in range(heads):
                     sc = (K[lo: pos + 1, h // group] @ q[t, h].double()) * scale
+                    if dist_bias is not None:
+                        dist = torch.clamp(pos - torch.arange(lo, pos + 1), max=dist_bias.shape[1] - 1)
+                        sc = sc + dist_bias[h].double()[dist]
                     p = torch.softmax(sc, dim=0)
                     out[t, h] = p @ V[lo: pos + 1, h // group]
         return out.reshape(n, heads * d).to(q.dtype)
