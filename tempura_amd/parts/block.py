@@ -104,6 +104,7 @@ class HyperConnection(Part):
     (``mix`` is indexed [from, to]).  Three small tensors, kept in float32."""
 
     category = "connection"
+    graph_safe = True      # three tensors read by kernels: nothing of the batch is seen on the host
 
     def __init__(self, spec, hidden_size, dtype, device):
         super().__init__(spec, hidden_size, dtype, device)
