@@ -58,7 +58,114 @@ def parse_args():
     ap.add_argument("--mixed-chunk", type=int, default=512)
     ap.add_argument("--mixed-temperature", type=float, default=0.0, help="0: greedy; above: seeded sampling with top-k 50")
     ap.add_argument("--decode-target-blocks", type=int, default=None, help="tuning: blocks the split decode attention aims at")
+    ap.add_argument("--design", default=None, choices=["mifutar"],
+                    help="instead of the headline: prefill and decode throughput of this design at layer sizes of real models, "
+                         "beside Llama layers of equal size, with the time of every kernel entry point")
+    ap.add_argument("--design-sizes", default="2048,4096", help="model widths of --design (comma separated)")
+    ap.add_argument("--design-layers", type=int, default=4, help="layers of each model of --design")
     return ap.parse_args()
+
+
+#: layer sizes of --design by model width: feed-forward width, attention heads x head size, key/value heads
+DESIGN_SIZES = {1024: (4096, 16, 64, 4), 2048: (8192, 32, 64, 8), 4096: (14336, 32, 128, 8), 8192: (28672, 64, 128, 8)}
+
+
+def design_bench(args) -> int:
+    """Prefill (one prompt, one step) and decode (a batch, captured steps) of the Mifutar design and of Llama layers
+    of the same width, feed-forward width and attention heads, random weights, bfloat16 unless --dtype says
+    otherwise.  A Mifutar model here has three state-space layers to one attention layer (window 1,024, four
+    streams); the Llama beside it has the same window.  Prints one JSON line."""
+    import torch
+    from tempura_amd.config import LlamaConfig, MifutarConfig
+    from tempura_amd.engine import Engine
+    from tempura_amd.engine.loading import random_model
+    from tempura_amd.engine.runner import StepEntry
+    from tempura_amd.kernels import ops
+
+    rng = random.Random(0)
+    window, vocab, T, batch = 1024, 32000, args.prompt_len, args.batch
+    points = {}
+
+    def say(msg):
+        print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+    def mifutar_config(width, ff, heads, dim, kv, layers):
+        mamba = {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}
+        attn = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "bias_max": 512,
+                "bias_buckets": 32, "mask": {"size": window}}
+        mlp = {"ff": ff, "kind": "dense", "limit": 7.0}
+        ls = [{"type": "attention", "mixer": attn, "mlp": mlp} if i % 4 == 3 else {"type": "mamba2", "mixer": mamba, "mlp": mlp}
+              for i in range(layers)]
+        return MifutarConfig.from_dict({"architecture": "Mifutar", "vocab": vocab, "width": width, "streams": 4, "logit_scale": 1.0,
+                                        "norm": {"eps": 1e-6}, "layers": ls, "max_positions": 8192})
+
+    def llama_config(width, ff, heads, dim, kv, layers):
+        return LlamaConfig(width, ff, layers, heads, kv, dim, vocab, 8192, 1e-5, 500000.0, None, False, sliding_window=window)
+
+    def measure(model):
+        pages = (batch + 1) * ((T + 600 + args.page_size - 1) // args.page_size) + 8
+        eng = Engine(model, dtype=args.dtype, page_size=args.page_size, kv_pages=pages, max_batch_size=batch + 1,
+                     max_num_batched_tokens=max(2048, T), use_graph=not args.no_graph)
+        runner = eng.runner
+        prompt = lambda n: [rng.randrange(vocab) for _ in range(n)]
+        times = []
+        for i in range(6):                        # prefill: a fresh request each time, the last four timed
+            rid = ("p", i)
+            runner.add_request(rid)
+            toks = prompt(T)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            runner.step([StepEntry(rid, toks, [T - 1])])
+            torch.cuda.synchronize()
+            if i >= 2:
+                times.append(time.perf_counter() - t)
+            runner.end_request(rid)
+        prefill_ms = 1e3 * sum(times) / len(times)
+        rids = [("d", i) for i in range(batch)]
+        for rid in rids:
+            runner.add_request(rid)
+            runner.step([StepEntry(rid, prompt(T), [])])
+        lg = runner.step([StepEntry(rid, [1], [0]) for rid in rids])
+        n_warm, n_steps = args.warmup, min(args.steps, 400)
+        for i in range(n_warm + n_steps):
+            if i == n_warm:
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+            toks = ops.argmax(lg).tolist()
+            lg = runner.step([StepEntry(rid, [tk], [0]) for rid, tk in zip(rids, toks)])
+        torch.cuda.synchronize()
+        decode_ms = 1e3 * (time.perf_counter() - t) / n_steps
+        for rid in rids:
+            runner.end_request(rid)
+        rep = eng.profile(prompt_len=T, batch=1, decode_steps=0)
+        rep_d = eng.profile(prompt_len=T, batch=batch, decode_steps=4)
+        table = lambda rows, div: {name: [calls // div if div > 1 else calls, round(us / div, 1)] for name, calls, us, _ in rows}
+        return {"prefill_tokens_per_s": round(T / (prefill_ms / 1e3), 1), "prefill_ms": round(prefill_ms, 3),
+                "decode_tokens_per_s": round(batch / (decode_ms / 1e3), 1), "decode_ms_per_step": round(decode_ms, 4),
+                "weight_bytes": model.weight_bytes(include_embedding=False),
+                "prefill_kernels_us": table(rep["prefill"], 1), "decode_kernels_us_per_step": table(rep_d["decode"], 4)}
+
+    for width in [int(w) for w in args.design_sizes.split(",") if w]:
+        if width not in DESIGN_SIZES:
+            print(f"--design-sizes: no layer sizes for width {width} (known: {sorted(DESIGN_SIZES)})", file=sys.stderr)
+            return 2
+        ff, heads, dim, kv = DESIGN_SIZES[width]
+        for name, cfg in (("mifutar", mifutar_config(width, ff, heads, dim, kv, args.design_layers)),
+                          ("llama", llama_config(width, ff, heads, dim, kv, args.design_layers))):
+            say(f"{name} width {width}: building")
+            model = random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
+            points[f"{name}_w{width}"] = measure(model)
+            say(f"{name} width {width}: prefill {points[f'{name}_w{width}']['prefill_tokens_per_s']} tok/s, "
+                f"decode {points[f'{name}_w{width}']['decode_tokens_per_s']} tok/s")
+            del model
+            torch.cuda.empty_cache()
+    first = f"mifutar_w{args.design_sizes.split(',')[0]}"
+    print(json.dumps({"metric": f"mifutar_prefill_tokens_per_s_T{T}", "value": points[first]["prefill_tokens_per_s"], "unit": "tokens/s",
+                      "n_gpus": 1, "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                      "data": "synthetic", "vs_baseline": None,
+                      "config": {"design": "Mifutar beside Llama layers of equal size", "layers": args.design_layers, "prompt": T,
+                                 "decode_batch": batch, "window": window}, "points": points}))
+    return 0
 
 
 def percentile(xs, p):
@@ -76,6 +183,12 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (this engine has no multi-GPU path); --gpus {args.gpus} is not supported")
         return 2
+    if args.design:
+        import torch
+        if not torch.cuda.is_available():
+            print("bench.py needs a GPU", file=sys.stderr)
+            return 3
+        return design_bench(args)
 
     import torch
     from tempura_amd.config import PRESETS, LlamaConfig

@@ -54,6 +54,9 @@ class AttentionMixer:
     scale: float
     bias_max: int
     window: Optional[int]
+    #: rows of the distance table.  The checkpoint's tensor says it; a configuration names it (``bias_buckets``)
+    #: only where no checkpoint is there to say it: for random weights
+    buckets: Optional[int] = None
 
     @classmethod
     def from_dict(cls, d, where):
@@ -65,7 +68,8 @@ class AttentionMixer:
             window = _num(mask, "size", where + ".mask")
         m = cls(_num(d, "heads", where), _num(d, "kv_heads", where), _num(d, "dim", where),
                 _num(d, "vdim", where) if d.get("vdim") is not None else _num(d, "dim", where),
-                _num(d, "scale", where, float), _num(d, "bias_max", where), window)
+                _num(d, "scale", where, float), _num(d, "bias_max", where), window,
+                _num(d, "bias_buckets", where) if d.get("bias_buckets") is not None else None)
         if m.heads % m.kv_heads != 0:
             raise ConfigError(f"config.json: {where}: heads ({m.heads}) must be a multiple of kv_heads ({m.kv_heads})")
         if m.vdim != m.dim:
@@ -77,6 +81,8 @@ class AttentionMixer:
              "bias_max": self.bias_max}
         if self.window is not None:
             d["mask"] = {"size": self.window}
+        if self.buckets is not None:
+            d["bias_buckets"] = self.buckets
         return d
 
 
@@ -261,7 +267,7 @@ class MifutarConfig:
                     "attention",
                     params={"num_heads": m.heads, "num_kv_heads": m.kv_heads, "head_dim": m.dim, "scale": m.scale,
                             "window": m.window, "position": PartSpec("none"), "values": "keys", "bias": True,
-                            "distance_bias": {"kind": "log_buckets", "max_distance": m.bias_max}},
+                            "distance_bias": {"kind": "log_buckets", "max_distance": m.bias_max, "buckets": m.buckets}},
                     weights={"q": f"{p}.mix.q", "k": f"{p}.mix.k", "o": f"{p}.mix.o", "q_bias": f"{p}.mix.q.b",
                              "k_bias": f"{p}.mix.k.b", "distance_bias": f"{p}.mix.rel"})
             else:

@@ -92,7 +92,8 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
                             int table_width, const int* cu_seqlens, const int* context_lens, void* out, int n_tokens,
                             int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale, int window,
                             int max_q_len, int num_single, int num_splits, float* scratch, const int* token_req,
-                            int portion_splits, int portion_min_steps, float* portion_scratch, hipStream_t s);
+                            int portion_splits, int portion_min_steps, float* portion_scratch, const float* dist_bias,
+                            int bias_len, hipStream_t s);
 
 extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, const void* v_cache,
                                   const int* block_tables, int table_width, const int* cu_seqlens,
@@ -114,11 +115,11 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
   TP_REQUIRE(n_heads <= 65535, "paged_attention: too many heads");
   if (n_tokens == 0) return 0;
   TP_REQUIRE(dist_bias == nullptr || bias_len > 0, "paged_attention: empty distance bias table");
-  if (dt == TP_BF16 && allow_fast && dist_bias == nullptr) {
+  if (dt == TP_BF16 && allow_fast) {
     const int rc = tp_paged_attention_fast(q, k_cache, v_cache, block_tables, table_width, cu_seqlens,
                                            context_lens, out, n_tokens, n_req, n_heads, n_kv, head_dim,
                                            page_size, scale, window, max_q_len, num_single, num_splits, scratch, token_req,
-                                           portion_splits, portion_min_steps, portion_scratch, s);
+                                           portion_splits, portion_min_steps, portion_scratch, dist_bias, bias_len, s);
     if (rc >= 0) return rc;
   }
   const dim3 grid(n_tokens, n_heads);

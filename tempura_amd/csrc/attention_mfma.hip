@@ -88,6 +88,10 @@ struct AttnArgs {
   int portion_min_steps;   // a query block is split into at most (its steps / this) parts
   float* portion_scratch;
   const int* token_req;
+  // a bias by distance, added to the scaled score (the scale does not multiply it): dist_bias [heads, bias_len]
+  // float32, entry min(query position - key position, bias_len - 1); nullptr: none
+  const float* dist_bias;
+  int bias_len;
 };
 #define PART_STRIDE(D) ((D) + 4)
 
@@ -164,9 +168,12 @@ __device__ inline void attn_scores(const bf16x8_t (&k)[2][D / 32], const bf16x8_
 
 // Softmax of one step's scores: probabilities as the next product's operand (pf), and the factor by
 // which the running sums shrink (alpha; `moved` false when no maximum of the wave moved: alpha is 1).
-template <int NQ, bool MASK>
+// BIAS: bias_row is this lane's row of the distance table (the row of its query column's head); the values
+// that are compared and exponentiated are then score * scale_log2 + bias * log2(e), formed before the maximum.
+template <int NQ, bool MASK, bool BIAS = false>
 __device__ inline void attn_softmax(const AttnArgs& a, int j0, const f32x4_t (&s)[NQ][2], const int (&qpos)[NQ],
-                                    float (&m)[NQ], float (&l)[NQ], bf16x8_t (&pf)[NQ], float (&alpha)[NQ], bool (&moved)[NQ]) {
+                                    float (&m)[NQ], float (&l)[NQ], bf16x8_t (&pf)[NQ], float (&alpha)[NQ], bool (&moved)[NQ],
+                                    const float* __restrict__ bias_row = nullptr) {
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;
 #pragma unroll
@@ -174,7 +181,23 @@ __device__ inline void attn_softmax(const AttnArgs& a, int j0, const f32x4_t (&s
     // this lane's keys: j0 + 8g + 4t + r
     float v[8];
     float mx = -INFINITY;
-    if (MASK) {
+    if (BIAS) {
+      const int hi = qpos[nq];
+      const int lo = a.window > 0 ? hi - a.window + 1 : 0;
+      float b[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {   // (all eight loads in flight; keys above the query read entry 0 and are masked)
+        const int key = j0 + 8 * g + 4 * (i >> 2) + (i & 3);
+        b[i] = bias_row[min(max(hi - key, 0), a.bias_len - 1)];
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = j0 + 8 * g + 4 * t + r;
+          v[t * 4 + r] = (key <= hi && key >= lo) ? fmaf(s[nq][t][r], a.scale_log2, b[t * 4 + r] * 1.4426950408889634f) : -INFINITY;
+        }
+    } else if (MASK) {
       const int hi = qpos[nq];
       const int lo = a.window > 0 ? hi - a.window + 1 : 0;
 #pragma unroll
@@ -193,12 +216,12 @@ __device__ inline void attn_softmax(const AttnArgs& a, int j0, const f32x4_t (&s
 #pragma unroll
     for (int i = 0; i < 8; ++i) mx = fmaxf(mx, v[i]);
     mx = quad_rows_max(mx);
-    const float m_new = fmaxf(m[nq], mx * a.scale_log2);    // the scale is positive
+    const float m_new = fmaxf(m[nq], BIAS ? mx : mx * a.scale_log2);    // the scale is positive
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column with nothing visible yet
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      v[i] = __builtin_amdgcn_exp2f(fmaf(v[i], a.scale_log2, -m_use));
+      v[i] = __builtin_amdgcn_exp2f(BIAS ? v[i] - m_use : fmaf(v[i], a.scale_log2, -m_use));
       sum += v[i];
     }
     u32x4_t pk;
@@ -300,36 +323,38 @@ __device__ inline void attn_pv(const bf16x8_t (&vf)[D / 16], const bf16x8_t (&pf
   }
 }
 
-template <int D, int NQ, bool MASK>
+template <int D, int NQ, bool MASK, bool BIAS = false>
 __device__ inline void attn_softmax_pv(const AttnArgs& a, int j0, const f32x4_t (&s)[NQ][2], const bf16x8_t (&vf)[D / 16],
-                                       const int (&qpos)[NQ], float (&m)[NQ], float (&l)[NQ], f32x4_t (&o)[NQ][D / 16]) {
+                                       const int (&qpos)[NQ], float (&m)[NQ], float (&l)[NQ], f32x4_t (&o)[NQ][D / 16],
+                                       const float* __restrict__ bias_row = nullptr) {
   bf16x8_t pf[NQ];
   float alpha[NQ];
   bool moved[NQ];
-  attn_softmax<NQ, MASK>(a, j0, s, qpos, m, l, pf, alpha, moved);
+  attn_softmax<NQ, MASK, BIAS>(a, j0, s, qpos, m, l, pf, alpha, moved, bias_row);
   attn_pv<D, NQ>(vf, pf, alpha, moved, o);
 }
 
-template <int D, int NQ, bool MASK = true>
+template <int D, int NQ, bool MASK = true, bool BIAS = false>
 __device__ inline void attn_compute(const AttnArgs& a, int j0, const KvFrags<D>& f, const bf16x8_t (&qf)[NQ][D / 32],
-                                    const int (&qpos)[NQ], float (&m)[NQ], float (&l)[NQ], f32x4_t (&o)[NQ][D / 16]) {
+                                    const int (&qpos)[NQ], float (&m)[NQ], float (&l)[NQ], f32x4_t (&o)[NQ][D / 16],
+                                    const float* __restrict__ bias_row = nullptr) {
   f32x4_t s[NQ][2];
   attn_scores<D, NQ>(f.k, qf, s);
-  attn_softmax_pv<D, NQ, MASK>(a, j0, s, f.v, qpos, m, l, o);
+  attn_softmax_pv<D, NQ, MASK, BIAS>(a, j0, s, f.v, qpos, m, l, o, bias_row);
 }
 
-template <int D, int NQ>
+template <int D, int NQ, bool BIAS = false>
 __device__ inline void attn_step(const AttnArgs& a, const int* __restrict__ table, int kvh, int ctx, int j0,
                                  const bf16x8_t (&qf)[NQ][D / 32], const int (&qpos)[NQ], float (&m)[NQ],
-                                 float (&l)[NQ], f32x4_t (&o)[NQ][D / 16]) {
+                                 float (&l)[NQ], f32x4_t (&o)[NQ][D / 16], const float* __restrict__ bias_row = nullptr) {
   KvFrags<D> f;
   attn_load<D>(a, table, kvh, ctx, j0, f);
-  attn_compute<D, NQ>(a, j0, f, qf, qpos, m, l, o);
+  attn_compute<D, NQ, true, BIAS>(a, j0, f, qf, qpos, m, l, o, bias_row);
 }
 
 // ---- prefill ----------------------------------------------------------------------------
 // grid: (query blocks of 16*NQ rows, kv_heads * ceil(group / 4), requests); block: 4 waves.
-template <int D, int NQ>
+template <int D, int NQ, bool BIAS = false>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int skip_single) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 4, c = lane & 15;
@@ -368,7 +393,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int skip_
   const int last_pos = pos0 + min(q0 + 16 * NQ, q_len) - 1;
   int first = 0;
   if (a.window > 0) first = max(0, pos0 + q0 - a.window + 1) & ~31;
-  for (int j0 = first; j0 <= last_pos; j0 += 32) attn_step<D, NQ>(a, table, kvh, ctx, j0, qf, qpos, m, l, o);
+  const float* bias_row = BIAS ? a.dist_bias + (size_t)head * a.bias_len : nullptr;
+  for (int j0 = first; j0 <= last_pos; j0 += 32) attn_step<D, NQ, BIAS>(a, table, kvh, ctx, j0, qf, qpos, m, l, o, bias_row);
 
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
@@ -749,7 +775,7 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
 // the requests fastest, 60 requests of 128 to 2,304 keys took 77 us where 60 of their mean took 54: the XCD
 // with the longest requests set the time, and more splits changed nothing, since the splits of a (request, head)
 // pair fell to the same XCD.)
-template <int D>
+template <int D, bool BIAS = false>
 __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   __shared__ float red_o[4][D][16];
   __shared__ float red_m[4][16], red_l[4][16];
@@ -785,7 +811,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   const int s_begin = blockIdx.z * per_split, s_end = min(steps, s_begin + per_split);
   // (Fetching the next step's fragments while this one is computed was measured: the doubled
   // fragment registers halve the occupancy and the kernel gets slower, not faster.)
-  for (int s = s_begin + wave; s < s_end; s += 4) attn_step<D, 1>(a, table, kvh, ctx, first + s * 32, qf, qpos, m, l, o);
+  const float* bias_row = BIAS ? a.dist_bias + (size_t)head * a.bias_len : nullptr;   // (a column is a head)
+  for (int s = s_begin + wave; s < s_end; s += 4) attn_step<D, 1, BIAS>(a, table, kvh, ctx, first + s * 32, qf, qpos, m, l, o, bias_row);
 
   // merge the four waves (fixed order), then write this split's partial
   float lt = l[0];
@@ -915,9 +942,13 @@ template <int D>
 static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int num_single, hipStream_t s) {
   const int group = a.n_heads / a.n_kv;
   const bool has_multi = num_single < n_req;
+  const bool bias = a.dist_bias != nullptr;
   if (num_single > 0) {
     const dim3 grid(a.n_kv * ((group + 15) / 16), n_req, a.num_splits);
-    hipLaunchKernelGGL(attn_decode_kernel<D>, grid, dim3(256), 0, s, a);
+    if (bias)
+      hipLaunchKernelGGL((attn_decode_kernel<D, true>), grid, dim3(256), 0, s, a);
+    else
+      hipLaunchKernelGGL(attn_decode_kernel<D>, grid, dim3(256), 0, s, a);
     if (a.num_splits > 1) {
       const dim3 cgrid(n_req, a.n_heads);
       hipLaunchKernelGGL(attn_combine_kernel, cgrid, dim3(64), 0, s, a.scratch, a.cu_seqlens, a.out, a.n_heads, D,
@@ -938,6 +969,16 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
     const bool two = g_attn_tune == 2 || (g_attn_tune != 3 && blocks2 >= 768);
     const int rows = two ? 32 : 16;
     const int skip = num_single > 0 ? 1 : 0;
+    if (bias) {
+      // (only the kernel whose waves load their own keys and values has the bias; it never splits a portion's keys)
+      a.portion_splits = 1;
+      const dim3 grid((max_q_len + rows - 1) / rows, kv_groups, n_req);
+      if (two)
+        hipLaunchKernelGGL((attn_prefill_kernel<D, 2, true>), grid, dim3(256), 0, s, a, skip);
+      else
+        hipLaunchKernelGGL((attn_prefill_kernel<D, 1, true>), grid, dim3(256), 0, s, a, skip);
+      return 0;
+    }
     if constexpr (D == 32 || D == 64 || D == 128) {
       if (a.portion_splits > 1 && g_attn_tune != 1 && a.page_shift >= 4 && a.page_size >= 512 / D) {
         // few query blocks under a long context: the keys of each are split over blocks (of 32 query rows)
@@ -973,7 +1014,8 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
                             int table_width, const int* cu_seqlens, const int* context_lens, void* out, int n_tokens,
                             int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale, int window,
                             int max_q_len, int num_single, int num_splits, float* scratch, const int* token_req,
-                            int portion_splits, int portion_min_steps, float* portion_scratch, hipStream_t s) {
+                            int portion_splits, int portion_min_steps, float* portion_scratch, const float* dist_bias,
+                            int bias_len, hipStream_t s) {
   if (head_dim % 32 != 0 || head_dim > 128 || page_size % 8 != 0) return -1;
   if (portion_min_steps < 1) return -1;
   if (portion_splits < 1 || portion_splits > 64 || (portion_splits > 1 && (portion_scratch == nullptr || token_req == nullptr))) return -1;
@@ -1003,6 +1045,9 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
   a.portion_min_steps = portion_min_steps;
   a.portion_scratch = portion_scratch;
   a.token_req = token_req;
+  a.dist_bias = dist_bias;
+  a.bias_len = bias_len;
+  if (dist_bias != nullptr && bias_len <= 0) return -1;
   a.scale_log2 = scale * 1.4426950408889634f;
   switch (head_dim) {
     case 32: launch_all<32>(a, n_tokens, n_req, max_q_len, num_single, s); break;

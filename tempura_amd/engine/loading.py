@@ -77,6 +77,13 @@ def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: 
                 # (rounded to the stored type as a written folder's norm weights are)
                 t = ops.fill_normal(t, _tensor_seed(seed, name), 1.0, norm_jitter).to(store).to(torch.float32)
             return t
+        if any(d is None for d in info.shape):
+            raise ValueError(f"tensor {name}: the configuration leaves a size to the checkpoint ({tuple(info.shape)}); "
+                             "random weights need it named")
+        if info.init in ("identity", "fraction"):
+            from ..weights.random_init import structured_mean
+            t = ops.fill_normal(torch.empty(info.shape, dtype=torch.float32, device=dev), _tensor_seed(seed, name), 0.0, std)
+            return (t + structured_mean(info).to(dev)).to(store)
         t = torch.empty(info.shape, dtype=parse_dtype(values_as) if values_as else store, device=dev)
         return ops.fill_normal(t, _tensor_seed(seed, name), 0.0, std).to(store)
 

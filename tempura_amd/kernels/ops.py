@@ -833,8 +833,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _dev_ok(dist_bias)
         _need(dist_bias.dtype == torch.float32 and dist_bias.dim() == 2 and dist_bias.shape[0] == heads and dist_bias.shape[1] > 0,
               "paged_attention: dist_bias must be float32 [heads, L]")
-    # (the matrix-core kernels have no distance bias)
-    fast = allow_fast_attention and q.dtype == torch.bfloat16 and d % 32 == 0 and d <= 128 and page_size % 8 == 0 and dist_bias is None
+    fast = allow_fast_attention and q.dtype == torch.bfloat16 and d % 32 == 0 and d <= 128 and page_size % 8 == 0
     splits, scratch = 1, None
     if fast and num_single > 0:
         # enough blocks to fill 256 CUs, but at least 128 keys per block
@@ -867,7 +866,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         if splits > 1:
             scratch = torch.empty((r * heads * splits * (d + 2),), dtype=torch.float32, device=q.device)
     parts, part_scratch = 1, None
-    if fast and num_single < r and d in (32, 64, 128) and page_size & (page_size - 1) == 0 and page_size >= max(8, 512 // d):
+    # (the kernel with a distance bias does not split a portion's keys)
+    if fast and dist_bias is None and num_single < r and d in (32, 64, 128) and page_size & (page_size - 1) == 0 and page_size >= max(8, 512 // d):
         # Few query blocks under a long context (a portion of a prompt behind a long cached prefix): the keys of
         # every portion are split over blocks until the chip is full (T = 512 behind 7,680 keys: 219 -> 137 us).
         q_blocks = -(-(n - num_single) // 32) + (r - num_single)

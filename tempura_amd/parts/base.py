@@ -21,7 +21,7 @@ class WeightInfo:
     """A tensor a part reads: its shape and how random-weight mode fills it."""
 
     shape: Tuple[int, ...]
-    init: str = "normal"          # "normal" (N(0, std)) or "ones"
+    init: str = "normal"          # "normal" (N(0, std)), "ones", "identity" (a square matrix: I + N(0, std)) or "fraction" (1 / n + N(0, std))
     optional: bool = False        # True: absence is legal (tied output head)
     kind: str = "float"           # "float": a weight (stored F32, BF16 or F16); "int": an integer table (kept as int32)
 

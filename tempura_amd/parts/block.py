@@ -114,7 +114,7 @@ class HyperConnection(Part):
     @classmethod
     def expected_weights(cls, spec, hidden_size):
         s, w = int(spec.params["streams"]), spec.weights
-        return {w["in"]: WeightInfo((s,)), w["out"]: WeightInfo((s,)), w["mix"]: WeightInfo((s, s))}
+        return {w["in"]: WeightInfo((s,), "fraction"), w["out"]: WeightInfo((s,), "ones"), w["mix"]: WeightInfo((s, s), "identity")}
 
     def load_weights(self, get):
         w = self.spec.weights

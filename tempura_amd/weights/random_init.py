@@ -46,6 +46,18 @@ def fill_normal_host(out: torch.Tensor, seed: int, mean: float, std: float) -> t
     return out
 
 
+def structured_mean(info: WeightInfo) -> torch.Tensor:
+    """What a tensor of init "identity" or "fraction" is drawn around (float32, on the host)."""
+    if info.init == "identity":
+        if len(info.shape) != 2 or info.shape[0] != info.shape[1]:
+            raise ValueError(f"init 'identity' needs a square matrix, got {tuple(info.shape)}")
+        return torch.eye(info.shape[0], dtype=torch.float32)
+    n = 1
+    for d in info.shape:
+        n *= int(d)
+    return torch.full(tuple(info.shape), 1.0 / max(1, n), dtype=torch.float32)
+
+
 def random_tensor(name: str, info: WeightInfo, seed: int, std: float, norm_jitter: float,
                   dtype: torch.dtype) -> torch.Tensor:
     """The tensor ``name`` of the random model with this seed.  Matrices are drawn in the stored type when
@@ -60,6 +72,9 @@ def random_tensor(name: str, info: WeightInfo, seed: int, std: float, norm_jitte
         if norm_jitter:
             fill_normal_host(t, key, 1.0, norm_jitter)
         return t.to(dtype)
+    if info.init in ("identity", "fraction"):
+        t = fill_normal_host(torch.empty(info.shape, dtype=torch.float32), key, 0.0, std)
+        return (t + structured_mean(info)).to(dtype)
     if dtype in (torch.float32, torch.bfloat16):
         return fill_normal_host(torch.empty(info.shape, dtype=dtype), key, 0.0, std)
     return fill_normal_host(torch.empty(info.shape, dtype=torch.float32), key, 0.0, std).to(dtype)

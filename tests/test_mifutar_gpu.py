@@ -174,9 +174,10 @@ def test_attention_with_distance_bias_and_a_key_that_stands_out(dtype, heads, kv
     token_req = torch.tensor([i for i, ql in enumerate(qlens) for _ in range(ql)], dtype=torch.int32)
     scale = d ** -0.5
     want = emu.paged_attention(q, kc, vc, tables, cu_t, ctx_t, token_req, scale, window, max(qlens), max(ctxs), dist_bias=bias)
-    got = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), tables.to(DEV), cu_t.to(DEV), ctx_t.to(DEV), token_req.to(DEV),
-                              scale, window, max(qlens), max(ctxs), num_single=0, dist_bias=bias.to(DEV))
-    _close(got, want, 2e-5 if dtype == torch.float32 else 2e-2)
+    for singles in (0, 3):        # every request as a portion; the single tokens through the kernel for decoding
+        got = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), tables.to(DEV), cu_t.to(DEV), ctx_t.to(DEV), token_req.to(DEV),
+                                  scale, window, max(qlens), max(ctxs), num_single=singles, dist_bias=bias.to(DEV))
+        _close(got, want, 2e-5 if dtype == torch.float32 else 2e-2)
     # and the stand-out key does decide where it is seen (the first request; the second has it one place outside)
     assert float((want.double()[cu[1] - 1]).abs().max()) > 2.0
     if window > 0 and ctxs[1] - 1 - window >= 0:
