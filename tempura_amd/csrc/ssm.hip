@@ -6,7 +6,7 @@
 //
 // A request r of the batch owns tokens cu_seqlens[r] .. cu_seqlens[r + 1] - 1 and the state row state_slots[r];
 // everything is read from device memory, so the same launches serve prompt portions, single decoded tokens and
-// captured steps.  Results do not depend on how a prompt was cut: the recurrence runs token by token in order.
+// captured steps.  How a prompt was cut changes rounding only.
 #include <math.h>
 
 #include "common.h"
@@ -83,10 +83,24 @@ extern "C" int tp_causal_conv(const float* in, int in_stride, int col0, const fl
 // xbc [n, channels] float32 holds, per token, x [heads * head_dim] | B [groups * state] | C [groups * state] (after
 // the convolution); dt_raw is column dt_col0 + h of the projection's rows.
 //
-// A block owns one request, one head and PC = 256 / R value columns; R lanes (a power of two, one part of a
-// wave) share a column and split the state index among them (n = lane + R i), NPT entries each in registers.
-// Tokens are taken TC at a time: their B, C, x, dt and decay are staged in LDS by all threads, then the run over
-// the chunk is register arithmetic, LDS broadcasts and one lane reduction per token.
+// A block owns one request, one head and PC = 256 / R value columns; R lanes (a power of two, neighbours in a
+// wave) share a column and split the state index among them, NPT consecutive entries each, in registers.
+// Tokens are taken TC at a time: their B, C, x, dt and decay are staged in LDS by all threads (rows padded with
+// zeros to R * NPT entries, so the run itself needs no bounds), then the run over the chunk is register
+// arithmetic, 16-byte LDS reads that most lanes share, and one reduction over the R lanes per token (row
+// permutes up to 16 lanes, which cost an instruction each and no trip through LDS).
+//
+// Long runs are cut into pieces of `piece` tokens that run side by side (a recurrence is a chain, and a prompt of
+// thousands of tokens on a chain leaves most of the chip idle).  Three launches of the same kernel:
+//   SCAN_LOCAL   every piece from a zero state: its end state and its total decay, to scratch;
+//   SCAN_CARRY   per (request, head, columns), piece by piece: the state a piece starts from is
+//                decay(previous piece) * (state the previous piece started from) + (its end state from zero);
+//                the state after the last piece is the request's new state;
+//   SCAN_OUTPUT  every piece again from the state it starts from, now writing y.
+// Short runs (single tokens above all) take SCAN_DIRECT: one launch, from the request's state to its new state.
+// How a run is cut changes rounding only.
+enum { SCAN_DIRECT = 0, SCAN_LOCAL = 1, SCAN_CARRY = 2, SCAN_OUTPUT = 3 };
+
 struct ScanArgs {
   const float* xbc;
   const float* proj;
@@ -101,42 +115,94 @@ struct ScanArgs {
   float* y;
   int heads, head_dim, n_state, groups, channels;
   int R, TC;
+  int mode, piece, max_pieces;
+  float* piece_state;   // [request, head, piece, n_state, head_dim]
+  float* piece_decay;   // [request, head, piece]
 };
+
+// sum over the R lanes (R a power of two, the lanes neighbours from a multiple of R on); every lane gets it
+__device__ inline float lanes_sum(float v, int R) {
+#define DPP_ADD(ctrl) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, false))
+  if (R >= 2) DPP_ADD(0xB1);    // quad_perm [1, 0, 3, 2]
+  if (R >= 4) DPP_ADD(0x4E);    // quad_perm [2, 3, 0, 1]
+  if (R >= 8) DPP_ADD(0x141);   // row_half_mirror: lane i of eight reads lane 7 - i
+  if (R >= 16) DPP_ADD(0x140);  // row_mirror: lane i of sixteen reads lane 15 - i
+#undef DPP_ADD
+  if (R >= 32) v += __shfl_xor(v, 16, TP_WAVE);
+  if (R >= 64) v += __shfl_xor(v, 32, TP_WAVE);
+  return v;
+}
 
 template <int NPT>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(ScanArgs a) {
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   const int N = a.n_state, P = a.head_dim, R = a.R, PC = 256 / a.R, TC = a.TC;
-  float* Bs = lds;                 // [TC, N]
-  float* Cs = Bs + (size_t)TC * N; // [TC, N]
-  float* xs = Cs + (size_t)TC * N; // [TC, PC]
+  const int NS = R * NPT;          // padded row of B and C
+  float* Bs = lds;                 // [TC, NS]
+  float* Cs = Bs + (size_t)TC * NS;
+  float* xs = Cs + (size_t)TC * NS; // [TC, PC]
   float* dts = xs + (size_t)TC * PC;
   float* das = dts + TC;
-  const int r = blockIdx.x, h = blockIdx.y, slice = blockIdx.z;
+  const int r = blockIdx.x, h = blockIdx.y;
+  const int slice = blockIdx.z % ((P + PC - 1) / PC), pc = blockIdx.z / ((P + PC - 1) / PC);
   const int col = threadIdx.x / R, rr = threadIdx.x % R;
   const int p = slice * PC + col;
   const bool active = p < P;
   const int g = h / (a.heads / a.groups);
-  const int start = a.cu_seqlens[r], len = a.cu_seqlens[r + 1] - start;
-  if (len <= 0) return;
+  const int run0 = a.cu_seqlens[r], run_len = a.cu_seqlens[r + 1] - run0;
+  if (run_len <= 0) return;
   const int inner = a.heads * P;
+  const int n0 = rr * NPT;
   float* S = a.state + (size_t)a.state_slots[r] * a.state_stride + a.state_off + (size_t)h * N * P;
+  const int pieces = a.mode == SCAN_DIRECT ? 1 : (run_len + a.piece - 1) / a.piece;
+  float* PS = a.piece_state + ((size_t)(r * a.heads + h) * a.max_pieces) * N * P;
+  float* PD = a.piece_decay + (size_t)(r * a.heads + h) * a.max_pieces;
+
+  if (a.mode == SCAN_CARRY) {
+    // the state each piece starts from, in place of what it ended with from zero; then the request's new state
+    float cur[NPT];
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) cur[i] = (active && n0 + i < N) ? S[(size_t)(n0 + i) * P + p] : 0.f;
+    for (int c = 0; c < pieces; ++c) {
+      const float decay = PD[c];
+      float* ps = PS + (size_t)c * N * P;
+#pragma unroll
+      for (int i = 0; i < NPT; ++i)
+        if (active && n0 + i < N) {
+          const float local = ps[(size_t)(n0 + i) * P + p];
+          ps[(size_t)(n0 + i) * P + p] = cur[i];
+          cur[i] = fmaf(decay, cur[i], local);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NPT; ++i)
+      if (active && n0 + i < N) S[(size_t)(n0 + i) * P + p] = cur[i];
+    return;
+  }
+  if (pc >= pieces) return;
+  const int start = a.mode == SCAN_DIRECT ? run0 : run0 + pc * a.piece;
+  const int len = a.mode == SCAN_DIRECT ? run_len : min(a.piece, run_len - pc * a.piece);
+  const float* init = a.mode == SCAN_DIRECT ? S : (a.mode == SCAN_OUTPUT ? PS + (size_t)pc * N * P : nullptr);
   float st[NPT];
 #pragma unroll
-  for (int i = 0; i < NPT; ++i) {
-    const int n = rr + R * i;
-    st[i] = (active && n < N) ? S[(size_t)n * P + p] : 0.f;
-  }
+  for (int i = 0; i < NPT; ++i) st[i] = (init != nullptr && active && n0 + i < N) ? init[(size_t)(n0 + i) * P + p] : 0.f;
   const float A = -expf(a.a_log[h]);
   const float dtb = a.dt_bias[h], Dh = a.d_skip[h];
+  const bool write_y = a.mode != SCAN_LOCAL;
+  float dt_sum = 0.f;
   for (int t0 = 0; t0 < len; t0 += TC) {
     const int nt = min(TC, len - t0);
     __syncthreads();
-    for (int idx = threadIdx.x; idx < nt * N; idx += 256) {
-      const int tt = idx / N, n = idx % N;
-      const float* row = a.xbc + (size_t)(start + t0 + tt) * a.channels + inner + g * N + n;
-      Bs[idx] = row[0];
-      Cs[idx] = row[(size_t)a.groups * N];
+    for (int idx = threadIdx.x; idx < nt * NS; idx += 256) {
+      const int tt = idx / NS, n = idx % NS;
+      float bv = 0.f, cv = 0.f;
+      if (n < N) {
+        const float* row = a.xbc + (size_t)(start + t0 + tt) * a.channels + inner + g * N + n;
+        bv = row[0];
+        cv = row[(size_t)a.groups * N];
+      }
+      Bs[idx] = bv;
+      Cs[idx] = cv;
     }
     for (int idx = threadIdx.x; idx < nt * PC; idx += 256) {
       const int tt = idx / PC, pp = slice * PC + idx % PC;
@@ -152,36 +218,65 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(ScanArgs a) {
       const float dt = dts[tt], da = das[tt];
       const float xv = xs[tt * PC + col];
       const float dx = dt * xv;
-      const float* Bt = Bs + (size_t)tt * N;
-      const float* Ct = Cs + (size_t)tt * N;
+      const float* Bt = Bs + (size_t)tt * NS + n0;
+      const float* Ct = Cs + (size_t)tt * NS + n0;
+      float bv[NPT], cv[NPT];
+      if constexpr (NPT % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < NPT; i += 4) {
+          const float4 b4 = *(const float4*)(Bt + i), c4 = *(const float4*)(Ct + i);
+          bv[i] = b4.x; bv[i + 1] = b4.y; bv[i + 2] = b4.z; bv[i + 3] = b4.w;
+          cv[i] = c4.x; cv[i + 1] = c4.y; cv[i + 2] = c4.z; cv[i + 3] = c4.w;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+          bv[i] = Bt[i];
+          cv[i] = Ct[i];
+        }
+      }
       float acc = 0.f;
 #pragma unroll
       for (int i = 0; i < NPT; ++i) {
-        const int n = rr + R * i;
-        if (n < N) {
-          st[i] = fmaf(da, st[i], dx * Bt[n]);
-          acc = fmaf(st[i], Ct[n], acc);
-        }
+        st[i] = fmaf(da, st[i], dx * bv[i]);
+        acc = fmaf(st[i], cv[i], acc);
       }
-      for (int o = R >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, TP_WAVE);
-      if (rr == 0 && active) a.y[(size_t)(start + t0 + tt) * inner + h * P + p] = fmaf(Dh, xv, acc);
+      dt_sum += dt;
+      if (write_y) {
+        acc = lanes_sum(acc, R);
+        if (rr == 0 && active) a.y[(size_t)(start + t0 + tt) * inner + h * P + p] = fmaf(Dh, xv, acc);
+      }
     }
   }
+  if (a.mode == SCAN_OUTPUT) return;
+  float* dst = a.mode == SCAN_DIRECT ? S : PS + (size_t)pc * N * P;
 #pragma unroll
-  for (int i = 0; i < NPT; ++i) {
-    const int n = rr + R * i;
-    if (active && n < N) S[(size_t)n * P + p] = st[i];
+  for (int i = 0; i < NPT; ++i)
+    if (active && n0 + i < N) dst[(size_t)(n0 + i) * P + p] = st[i];
+  if (a.mode == SCAN_LOCAL && slice == 0 && threadIdx.x == 0) PD[pc] = expf(A * dt_sum);
+}
+
+// scratch floats a scan of n_req requests whose longest run has max_run tokens needs (0: it runs in one launch)
+extern "C" size_t tp_ssm_scan_scratch(int n_req, int max_run, int heads, int head_dim, int n_state, int* piece_out) {
+  int piece = 0;
+  if (max_run > 256) {
+    piece = 128;
+    while ((max_run + piece - 1) / piece > 32) piece *= 2;    // at most 32 pieces a run
   }
+  if (piece_out) *piece_out = piece;
+  if (piece == 0) return 0;
+  const size_t pieces = (size_t)((max_run + piece - 1) / piece);
+  return (size_t)n_req * heads * pieces * ((size_t)n_state * head_dim + 1);
 }
 
 extern "C" int tp_ssm_scan(const float* xbc, const float* proj, int proj_stride, int dt_col0, const float* dt_bias,
                            const float* a_log, const float* d_skip, float* state, size_t state_stride, size_t state_off,
                            const int* cu_seqlens, const int* state_slots, float* y, int n_req, int heads, int head_dim,
-                           int n_state, int groups, hipStream_t s) {
+                           int n_state, int groups, int max_run, float* scratch, size_t scratch_floats, hipStream_t s) {
   TP_REQUIRE(n_req >= 0 && heads > 0 && head_dim > 0 && n_state > 0 && groups > 0 && heads % groups == 0, "ssm_scan: bad sizes");
   TP_REQUIRE(n_state <= 1024, "ssm_scan: state size %d exceeds 1024", n_state);
   TP_REQUIRE(state_stride >= state_off + (size_t)heads * n_state * head_dim, "ssm_scan: state rows too short");
-  TP_REQUIRE(heads <= 65535, "ssm_scan: too many heads");
+  TP_REQUIRE(heads <= 65535 && max_run >= 0, "ssm_scan: too many heads");
   if (n_req == 0) return 0;
   ScanArgs a;
   a.xbc = xbc; a.proj = proj; a.proj_stride = proj_stride; a.dt_col0 = dt_col0;
@@ -197,22 +292,45 @@ extern "C" int tp_ssm_scan(const float* xbc, const float* proj, int proj_stride,
   int pc_pow2 = 1;
   while (pc_pow2 < head_dim) pc_pow2 *= 2;
   while (R < 64 && 256 / R > pc_pow2) R *= 2;
-  const int npt = (n_state + R - 1) / R;
+  const int per_lane = (n_state + R - 1) / R;
+  const int npt = per_lane <= 1 ? 1 : (per_lane <= 2 ? 2 : (per_lane <= 4 ? 4 : (per_lane <= 8 ? 8 : 16)));
   a.R = R;
   const int PC = 256 / R;
-  const int per_token = 2 * n_state + PC + 2;
+  const int per_token = 2 * R * npt + PC + 2;
   int TC = (32 * 1024 / 4) / per_token;
   TC = TC < 1 ? 1 : (TC > 64 ? 64 : TC);
   a.TC = TC;
   const size_t shmem = (size_t)TC * per_token * sizeof(float);
-  const dim3 grid(n_req, heads, (head_dim + PC - 1) / PC);
-  TP_REQUIRE(grid.z <= 65535, "ssm_scan: head_dim too large");
-#define SCAN_LAUNCH(NPT) hipLaunchKernelGGL(ssm_scan_kernel<NPT>, grid, dim3(256), shmem, s, a)
-  if (npt <= 1) SCAN_LAUNCH(1);
-  else if (npt <= 2) SCAN_LAUNCH(2);
-  else if (npt <= 4) SCAN_LAUNCH(4);
-  else if (npt <= 8) SCAN_LAUNCH(8);
-  else SCAN_LAUNCH(16);
+  const int slices = (head_dim + PC - 1) / PC;
+  int piece = 0;
+  const size_t need = tp_ssm_scan_scratch(n_req, max_run, heads, head_dim, n_state, &piece);
+  a.piece = piece;
+  a.max_pieces = piece ? (max_run + piece - 1) / piece : 1;
+  a.piece_state = scratch;
+  a.piece_decay = scratch ? scratch + (size_t)n_req * heads * a.max_pieces * n_state * head_dim : nullptr;
+  TP_REQUIRE(piece == 0 || (scratch != nullptr && scratch_floats >= need), "ssm_scan: scratch of %zu floats needed", need);
+  TP_REQUIRE((long)slices * a.max_pieces <= 65535, "ssm_scan: too many pieces");
+#define SCAN_LAUNCH(NPT, GRID) hipLaunchKernelGGL(ssm_scan_kernel<NPT>, GRID, dim3(256), shmem, s, a)
+#define SCAN_DISPATCH(GRID)            \
+  do {                                 \
+    if (npt == 1) SCAN_LAUNCH(1, GRID);      \
+    else if (npt == 2) SCAN_LAUNCH(2, GRID); \
+    else if (npt == 4) SCAN_LAUNCH(4, GRID); \
+    else if (npt == 8) SCAN_LAUNCH(8, GRID); \
+    else SCAN_LAUNCH(16, GRID);              \
+  } while (0)
+  if (piece == 0) {
+    a.mode = SCAN_DIRECT;
+    SCAN_DISPATCH(dim3(n_req, heads, slices));
+  } else {
+    a.mode = SCAN_LOCAL;
+    SCAN_DISPATCH(dim3(n_req, heads, slices * a.max_pieces));
+    a.mode = SCAN_CARRY;
+    SCAN_DISPATCH(dim3(n_req, heads, slices));
+    a.mode = SCAN_OUTPUT;
+    SCAN_DISPATCH(dim3(n_req, heads, slices * a.max_pieces));
+  }
+#undef SCAN_DISPATCH
 #undef SCAN_LAUNCH
   TP_CHECK_LAUNCH("ssm_scan");
   return 0;

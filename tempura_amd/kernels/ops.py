@@ -309,12 +309,13 @@ def causal_conv(proj: torch.Tensor, col0: int, channels: int, weight: torch.Tens
 
 def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col0: int, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
              state: torch.Tensor, state_off: int, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, num_requests: int,
-             num_heads: int, head_dim: int, state_size: int, groups: int) -> torch.Tensor:
+             num_heads: int, head_dim: int, state_size: int, groups: int, max_run: Optional[int] = None) -> torch.Tensor:
     """The selective recurrence per head over each request's run: with dt = softplus(proj[:, dt_col0 + h] + dt_bias[h])
     and a = exp(-exp(a_log[h]) * dt):  S <- a S + dt B x^T,  y = S^T C + d_skip[h] x.  ``xbc`` float32 [n, channels]
     holds x [heads * head_dim] | B [groups * state] | C [groups * state]; the state [heads, state, head_dim] of a
     request lives at ``state[slot, state_off:]`` (float32), is read at the start of the run and left as the run
-    leaves it.  Returns y float32 [n, heads * head_dim]."""
+    leaves it.  ``max_run``: the longest run of the batch (None: the number of rows); long runs are cut into
+    pieces that run side by side, which changes rounding only.  Returns y float32 [n, heads * head_dim]."""
     if _backend is not None:
         return _backend.ssm_scan(xbc, proj, dt_col0, dt_bias, a_log, d_skip, state, state_off, cu_seqlens, state_slots,
                                  num_requests, num_heads, head_dim, state_size, groups)
@@ -333,9 +334,14 @@ def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col0: int, dt_bias: torch
     _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
     _i32(state_slots, num_requests, "state_slots")
     y = torch.empty((n, inner), dtype=torch.float32, device=xbc.device)
+    max_run = n if max_run is None else min(int(max_run), n)
+    lib = _Library.get()
+    lib.tp_ssm_scan_scratch.restype = ctypes.c_size_t
+    need = lib.tp_ssm_scan_scratch(int(num_requests), max_run, num_heads, head_dim, state_size, None)
+    scratch = torch.empty((need,), dtype=torch.float32, device=xbc.device) if need else None
     _call("tp_ssm_scan", _ptr(xbc), _ptr(proj), proj.shape[1], int(dt_col0), _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(state),
           ctypes.c_size_t(state.shape[1]), ctypes.c_size_t(state_off), _ptr(cu_seqlens), _ptr(state_slots), _ptr(y),
-          int(num_requests), num_heads, head_dim, state_size, groups, _stream())
+          int(num_requests), num_heads, head_dim, state_size, groups, max_run, _ptr(scratch), ctypes.c_size_t(need), _stream())
     return y
 
 

@@ -87,7 +87,7 @@ class Mamba2Mixer(Mixer):
                               ctx.token_req, ctx.state_slots, ctx.num_requests)
         y = ops.ssm_scan(xbc, proj, self.inner + self.channels, self.dt_bias, self.a_log, self.d_skip, cache.state,
                          self.conv_state, ctx.cu_seqlens, ctx.state_slots, ctx.num_requests, self.num_heads, self.head_dim,
-                         self.state_size, self.groups)
+                         self.state_size, self.groups, max_run=ctx.max_q_len)
         v = ops.gated_group_norm(y, proj, 0, self.norm_w, self.norm_eps, self.norm_groups, self.dtype)
         return ops.linear(v, self.w_out, torch.float32, residual=residual)
 

@@ -87,7 +87,7 @@ class EmuOps:
         return (out * torch.sigmoid(out)).to(torch.float32)
 
     def ssm_scan(self, xbc, proj, dt_col0, dt_bias, a_log, d_skip, state, state_off, cu_seqlens, state_slots, num_requests,
-                 num_heads, head_dim, state_size, groups):
+                 num_heads, head_dim, state_size, groups, max_run=None):
         n = xbc.shape[0]
         H, P, N, G = num_heads, head_dim, state_size, groups
         inner = H * P

@@ -240,6 +240,30 @@ def test_selective_scan_and_its_state(H, P, N, G):
     assert torch.equal(torch.cat([ya, yb]), got[:70]) and torch.equal(s_two[2], s_dev[2])
 
 
+@pytest.mark.parametrize("H,P,N,G", [(4, 8, 16, 2), (3, 40, 24, 1), (8, 64, 128, 4)])
+def test_long_runs_in_pieces_side_by_side(H, P, N, G):
+    """Runs long enough to be cut into pieces that run side by side, beside short ones and a single token, from states
+    that are not zero: the same result as token by token, up to rounding."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(H + N)
+    inner, ch = H * P, H * P + 2 * G * N
+    runs = [700, 1, 300, 2, 129]
+    n = sum(runs)
+    cu = torch.tensor([0, 700, 701, 1001, 1003, 1132], dtype=torch.int32)
+    slots = torch.tensor([1, 4, 0, 3, 2], dtype=torch.int32)
+    state = torch.randn(6, 5 + H * N * P, generator=g) * 0.5
+    xbc = torch.randn(n, ch, generator=g) * 0.7
+    proj = torch.randn(n, H + 2, generator=g)
+    dt_bias, a_log, d_skip = torch.randn(H, generator=g) - 1.5, torch.log(torch.rand(H, generator=g) * 0.5 + 0.05), torch.randn(H, generator=g)
+    s_ref, s_dev = state.clone(), state.to(DEV)
+    want = emu.ssm_scan(xbc, proj, 1, dt_bias, a_log, d_skip, s_ref, 5, cu, slots, 5, H, P, N, G)
+    got = ops.ssm_scan(xbc.to(DEV), proj.to(DEV), 1, dt_bias.to(DEV), a_log.to(DEV), d_skip.to(DEV), s_dev, 5, cu.to(DEV),
+                       slots.to(DEV), 5, H, P, N, G, max_run=700)
+    _close(got, want, 2e-5)
+    _close(s_dev, s_ref, 2e-5)
+    assert torch.equal(s_dev.cpu()[5], state[5]) and torch.equal(s_dev.cpu()[:, :5], state[:, :5])
+
+
 @pytest.mark.parametrize("inner,groups", [(32, 1), (48, 3), (288, 2), (4096, 4)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 def test_gated_group_norm(inner, groups, out_dtype):
