@@ -193,20 +193,23 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(ScanArgs a) {
   for (int t0 = 0; t0 < len; t0 += TC) {
     const int nt = min(TC, len - t0);
     __syncthreads();
-    for (int idx = threadIdx.x; idx < nt * NS; idx += 256) {
-      const int tt = idx / NS, n = idx % NS;
-      float bv = 0.f, cv = 0.f;
-      if (n < N) {
-        const float* row = a.xbc + (size_t)(start + t0 + tt) * a.channels + inner + g * N + n;
-        bv = row[0];
-        cv = row[(size_t)a.groups * N];
+    // (a wave stages every fourth token, its lanes the entries of a row: no division in the loop)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int tt = wave; tt < nt; tt += 4) {
+      const float* row = a.xbc + (size_t)(start + t0 + tt) * a.channels;
+      for (int n = lane; n < NS; n += 64) {
+        float bv = 0.f, cv = 0.f;
+        if (n < N) {
+          bv = row[inner + g * N + n];
+          cv = row[inner + (a.groups + g) * N + n];
+        }
+        Bs[tt * NS + n] = bv;
+        Cs[tt * NS + n] = cv;
       }
-      Bs[idx] = bv;
-      Cs[idx] = cv;
-    }
-    for (int idx = threadIdx.x; idx < nt * PC; idx += 256) {
-      const int tt = idx / PC, pp = slice * PC + idx % PC;
-      xs[idx] = pp < P ? a.xbc[(size_t)(start + t0 + tt) * a.channels + h * P + pp] : 0.f;
+      for (int c = lane; c < PC; c += 64) {
+        const int pp = slice * PC + c;
+        xs[tt * PC + c] = pp < P ? row[h * P + pp] : 0.f;
+      }
     }
     for (int idx = threadIdx.x; idx < nt; idx += 256) {
       const float dt = softplus_f(a.proj[(size_t)(start + t0 + idx) * a.proj_stride + a.dt_col0 + h] + dtb);
@@ -274,7 +277,7 @@ extern "C" int tp_ssm_scan(const float* xbc, const float* proj, int proj_stride,
                            const int* cu_seqlens, const int* state_slots, float* y, int n_req, int heads, int head_dim,
                            int n_state, int groups, int max_run, float* scratch, size_t scratch_floats, hipStream_t s) {
   TP_REQUIRE(n_req >= 0 && heads > 0 && head_dim > 0 && n_state > 0 && groups > 0 && heads % groups == 0, "ssm_scan: bad sizes");
-  TP_REQUIRE(n_state <= 1024, "ssm_scan: state size %d exceeds 1024", n_state);
+  TP_REQUIRE(n_state <= 2048, "ssm_scan: state size %d exceeds 2048", n_state);
   TP_REQUIRE(state_stride >= state_off + (size_t)heads * n_state * head_dim, "ssm_scan: state rows too short");
   TP_REQUIRE(heads <= 65535 && max_run >= 0, "ssm_scan: too many heads");
   if (n_req == 0) return 0;
@@ -285,15 +288,16 @@ extern "C" int tp_ssm_scan(const float* xbc, const float* proj, int proj_stride,
   a.cu_seqlens = cu_seqlens; a.state_slots = state_slots; a.y = y;
   a.heads = heads; a.head_dim = head_dim; a.n_state = n_state; a.groups = groups;
   a.channels = heads * head_dim + 2 * groups * n_state;
-  // lanes per column: enough that a lane holds at most 8 state entries (16 beyond 512), and no more columns than
-  // the head has values
+  // lanes per column: enough that a lane holds at most 32 state entries, and no more columns than the head has
+  // values.  Few lanes a column and many entries a lane: the B and C rows a block stages serve more columns, and
+  // more of a wave's instructions are the recurrence's own.
   int R = 1;
-  while (R < 64 && R * 8 < n_state) R *= 2;
+  while (R < 64 && R * 32 < n_state) R *= 2;
   int pc_pow2 = 1;
   while (pc_pow2 < head_dim) pc_pow2 *= 2;
   while (R < 64 && 256 / R > pc_pow2) R *= 2;
   const int per_lane = (n_state + R - 1) / R;
-  const int npt = per_lane <= 1 ? 1 : (per_lane <= 2 ? 2 : (per_lane <= 4 ? 4 : (per_lane <= 8 ? 8 : 16)));
+  const int npt = per_lane <= 1 ? 1 : (per_lane <= 2 ? 2 : (per_lane <= 4 ? 4 : (per_lane <= 8 ? 8 : (per_lane <= 16 ? 16 : 32))));
   a.R = R;
   const int PC = 256 / R;
   const int per_token = 2 * R * npt + PC + 2;
@@ -317,7 +321,8 @@ extern "C" int tp_ssm_scan(const float* xbc, const float* proj, int proj_stride,
     else if (npt == 2) SCAN_LAUNCH(2, GRID); \
     else if (npt == 4) SCAN_LAUNCH(4, GRID); \
     else if (npt == 8) SCAN_LAUNCH(8, GRID); \
-    else SCAN_LAUNCH(16, GRID);              \
+    else if (npt == 16) SCAN_LAUNCH(16, GRID); \
+    else SCAN_LAUNCH(32, GRID);              \
   } while (0)
   if (piece == 0) {
     a.mode = SCAN_DIRECT;

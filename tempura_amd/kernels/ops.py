@@ -330,7 +330,7 @@ def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col0: int, dt_bias: torch
         _need(t.dtype == torch.float32 and t.numel() == num_heads, "ssm_scan: per-head constants must be float32 [heads]")
     _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= state_off + num_heads * state_size * head_dim,
           "ssm_scan: state rows too short")
-    _need(num_heads % groups == 0 and state_size <= 1024, "ssm_scan: heads must be a multiple of groups, state size at most 1024")
+    _need(num_heads % groups == 0 and state_size <= 2048, "ssm_scan: heads must be a multiple of groups, state size at most 2048")
     _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
     _i32(state_slots, num_requests, "state_slots")
     y = torch.empty((n, inner), dtype=torch.float32, device=xbc.device)
