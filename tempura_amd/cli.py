@@ -147,15 +147,14 @@ def cmd_inspect(args) -> int:
 
 
 def cmd_random_model(args) -> int:
-    from .config import PRESETS, LlamaConfig
+    from .config import PRESETS, LlamaConfig, config_from_file
     from .weights import write_random_model
     if args.list:
         for name, cfg in sorted(PRESETS.items()):
             print(f"{name}: {cfg.num_hidden_layers} layers, hidden {cfg.hidden_size}, {cfg.num_parameters() / 1e6:.1f} M parameters")
         return 0
     if args.config_json:
-        with open(args.config_json) as f:
-            cfg = LlamaConfig.from_json(f.read())
+        cfg = config_from_file(args.config_json)      # (any registered architecture, chosen by what the file names)
     elif args.model_config in PRESETS:
         cfg = LlamaConfig.from_dict(PRESETS[args.model_config].to_dict())
     else:
@@ -168,7 +167,7 @@ def cmd_random_model(args) -> int:
 
 
 def main(argv=None) -> int:
-    ap = argparse.ArgumentParser(prog="tempura", description="Llama 3 inference on one MI355X")
+    ap = argparse.ArgumentParser(prog="tempura", description="Decoder-only language models (Llama 3, Mifutar) on one MI355X")
     sub = ap.add_subparsers(dest="cmd", required=True)
 
     p = sub.add_parser("inspect", help="print what a model folder holds")

@@ -241,7 +241,7 @@ class MifutarConfig:
         for info in expected_weights(self.build_spec()).values():
             n = 1
             for s in info.shape:
-                n *= int(s)
+                n *= int(s) if s is not None else 0      # (a size only the checkpoint says: not counted)
             total += n
         return total
 
@@ -255,6 +255,22 @@ class MifutarConfig:
                 m = l.mixer
                 total += 4 * (m.heads * m.state * m.vdim + (m.conv - 1) * (m.heads * m.vdim + 2 * m.groups * m.state))
         return total
+
+    def describe(self) -> Dict[str, Any]:
+        """What ``tempura inspect`` prints of this architecture."""
+        def layer(l):
+            m = l.mixer
+            if l.type == "attention":
+                mix = (f"attention {m.heads} heads ({m.kv_heads} key/value) of {m.dim}, window {m.window or 'none'}, "
+                       f"distance bias up to {m.bias_max}")
+            else:
+                mix = (f"mamba2 {m.heads} heads of {m.vdim}, state {m.state}, {m.groups} groups, {m.conv} taps, "
+                       f"norm in {m.norm_groups} parts")
+            return mix + (f"; feed-forward {l.mlp.ff}, limit {l.mlp.limit:g}" if l.mlp is not None else "; no feed-forward")
+        return {"hidden_size": self.width, "vocab_size": self.vocab, "streams": self.streams or 1,
+                "logit_scale": self.logit_scale, "norm_eps": self.norm_eps, "max_positions": self.max_positions,
+                "layers": [layer(l) for l in self.layers],
+                "kv_bytes_per_token_bf16": self.kv_bytes_per_token(2), "state_bytes_per_request": self.state_bytes_per_request()}
 
     def build_spec(self) -> ModelSpec:
         layers = []

@@ -40,7 +40,12 @@ def config_class_for(name: str):
 
 def load_config(model_dir: str):
     """Read ``model_dir/config.json`` and return the typed config its architecture names."""
-    path = os.path.join(model_dir, "config.json")
+    return config_from_file(os.path.join(model_dir, "config.json"))
+
+
+def config_from_file(path: str):
+    """The typed config of a config.json file, by the architecture it names (``architectures``, ``model_type`` or
+    ``architecture``)."""
     try:
         with open(path, "r") as f:
             text = f.read()

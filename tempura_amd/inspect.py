@@ -18,13 +18,25 @@ from .weights.safetensors_io import SafetensorsFile
 def inspect(model_dir: str) -> Dict[str, Any]:
     cfg = load_config(model_dir)
     files = sorted(glob.glob(os.path.join(model_dir, "*.safetensors")))
-    n_tensors, size, dtypes = 0, 0, set()
+    n_tensors, size, dtypes, stored = 0, 0, set(), 0
     for p in files:
         f = SafetensorsFile(p)
         n_tensors += len(f.names())
+        for n in f.names():
+            count = 1
+            for d in f.shape(n):
+                count *= int(d)
+            stored += count
         dtypes.update(f.dtype_tag(n) for n in f.names())
         size += os.path.getsize(p)
         f.close()
+    if hasattr(cfg, "describe"):
+        # an architecture that describes itself: its own fields beside the ones every folder has
+        info = {"format": "safetensors" if files else "none", "architecture": cfg.architecture}
+        info.update(cfg.describe())
+        info.update({"dtypes": sorted(dtypes), "tensors": n_tensors, "size_bytes": size,
+                     "parameters": stored if files else cfg.num_parameters()})
+        return info
     rs = cfg.rope_scaling
     return {
         "format": "safetensors" if files else "none",
@@ -52,6 +64,21 @@ def inspect(model_dir: str) -> Dict[str, Any]:
 
 
 def format_report(info: Dict[str, Any]) -> str:
+    if "kv_heads" not in info:
+        # a self-described architecture: one line per field, lists one entry a line
+        lines = []
+        for k, v in info.items():
+            label = k.replace("_", " ").capitalize() + ":"
+            if isinstance(v, list) and k == "layers":
+                lines.append(label)
+                lines.extend(f"  {i:3d}  {e}" for i, e in enumerate(v))
+            elif k == "size_bytes":
+                lines.append(f"{'Size:':17s}{v / 1e6:.1f} MB")
+            elif k == "parameters":
+                lines.append(f"{'Parameters:':17s}{v / 1e6:.2f} M")
+            else:
+                lines.append(f"{label:17s}{', '.join(v) if isinstance(v, list) else v}")
+        return "\n".join(lines)
     gqa = "MHA" if info["kv_heads"] == info["attention_heads"] else ("MQA" if info["kv_heads"] == 1 else "GQA")
     lines = [
         f"Format:          {info['format']}",

@@ -230,3 +230,23 @@ def test_engine_generates_what_plain_greedy_generates(dirs, name):
     outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=6))
     for p, o in zip(prompts, outs):
         assert o == plain.greedy(cfg, W, p, 6)
+
+
+def test_command_line_inspects_and_writes_random_folders(dirs, tmp_path, capsys):
+    """`tempura inspect` on a folder of the design, and `tempura random-model --config-json` for it (the rows of
+    the distance table named in the file, since no checkpoint is there to say them)."""
+    from tempura_amd.cli import main
+    from tempura_amd.engine.loading import load_model
+    assert main(["inspect", dirs["mix"]]) == 0
+    text = capsys.readouterr().out
+    assert "Mifutar" in text and "mamba2 4 heads of 8" in text and "window 7" in text
+    cfg = cases.config_json("attn")
+    for layer, rows in zip(cfg["layers"], (8, 4, 10)):
+        layer["mixer"]["bias_buckets"] = rows
+    path = tmp_path / "c.json"
+    path.write_text(json.dumps(cfg))
+    assert main(["random-model", "--config-json", str(path), "--out", str(tmp_path / "rnd"), "--std", "0.3"]) == 0
+    model = load_model(str(tmp_path / "rnd"), "float32", "cpu")
+    assert model.layers[2].mixer.dist_table.shape[0] == 6 and model.streams == 1
+    # connection tensors are drawn around the plain residual sum
+    assert abs(float(model.layers[0].mixer_link.mix[0, 0]) - 1.0) < 1.5
