@@ -170,10 +170,11 @@ __device__ inline void attn_scores(const bf16x8_t (&k)[2][D / 32], const bf16x8_
 // which the running sums shrink (alpha; `moved` false when no maximum of the wave moved: alpha is 1).
 // BIAS: bias_row is this lane's row of the distance table (the row of its query column's head); the values
 // that are compared and exponentiated are then score * scale_log2 + bias * log2(e), formed before the maximum.
-template <int NQ, bool MASK, bool BIAS = false>
+// (BP: a pointer to global memory, or to LDS where a kernel keeps its heads' rows there)
+template <int NQ, bool MASK, bool BIAS = false, typename BP = const float*>
 __device__ inline void attn_softmax(const AttnArgs& a, int j0, const f32x4_t (&s)[NQ][2], const int (&qpos)[NQ],
                                     float (&m)[NQ], float (&l)[NQ], bf16x8_t (&pf)[NQ], float (&alpha)[NQ], bool (&moved)[NQ],
-                                    const float* __restrict__ bias_row = nullptr) {
+                                    BP bias_row = nullptr) {
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;
 #pragma unroll
@@ -444,8 +445,13 @@ __device__ __host__ inline int portion_parts(int steps, int max_parts, int min_s
   return max_parts <= 1 ? 1 : min(max_parts, max(1, steps / min_steps));
 }
 
-template <int D, int NQ, int NS = 4, int OCC = 2>
+#define ATTN_BIAS_LDS 1024   // the longest distance table a wave keeps in LDS
+template <int D, int NQ, int NS = 4, int OCC = 2, bool BIAS = false>
 __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, int skip_single) {
+  static_assert(!BIAS || NQ == 1, "the distance bias is in the variant of one query tile a wave");
+  // (each wave's head has its row of the distance table in LDS: a load from global memory inside the loop would
+  // have to wait for every copy into LDS that is in flight)
+  __shared__ float bias_lds[BIAS ? 4 * ATTN_BIAS_LDS : 1];
   constexpr int C = D / 8;             // 16-byte chunks per key row
   constexpr int SH = C == 16 ? 0 : (C == 8 ? 1 : 2);
   constexpr int KI = D / 16;           // 1 KB loads per key tile (32 rows of 2 D bytes), and per value tile
@@ -506,6 +512,12 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
     nsteps = s_end - s_begin;
   }
   const int qpos_min = pos0 + min(q0, q_len - 1);   // the earliest query of this block
+  if constexpr (BIAS) {
+    for (int i = lane; i < a.bias_len; i += 64) bias_lds[wave * ATTN_BIAS_LDS + i] = a.dist_bias[(size_t)head * a.bias_len + i];
+    __syncthreads();
+  }
+  typedef const __attribute__((address_space(3))) float* lds_row_t;
+  const lds_row_t bias_row = (lds_row_t)&bias_lds[BIAS ? wave * ATTN_BIAS_LDS : 0];
 
   // What this lane fetches in each of its loads of a step: load t = wave + 4 i.  t < KI is a piece of the key tile
   // (64 chunk slots: 64 / C whole rows of one group of eight keys), else a piece of the value tile: the step's keys
@@ -706,7 +718,9 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
         attn_scores<D, NQ>(kf, qf, nxt);
       }
       ATTN_RV(0); ATTN_RV(1); ATTN_RV(2); ATTN_RV(3); ATTN_RV(4); ATTN_RV(5); ATTN_RV(6); ATTN_RV(7);
-      if (plain_step)
+      if constexpr (BIAS)
+        attn_softmax<NQ, true, true, lds_row_t>(a, j0, cur, qpos, m, l, pf, alpha, moved, bias_row);
+      else if (plain_step)
         attn_softmax<NQ, false>(a, j0, cur, qpos, m, l, pf, alpha, moved);
       else
         attn_softmax<NQ, true>(a, j0, cur, qpos, m, l, pf, alpha, moved);
@@ -972,6 +986,14 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
     if (bias) {
       // (only the kernel whose waves load their own keys and values has the bias; it never splits a portion's keys)
       a.portion_splits = 1;
+      if constexpr (D == 32 || D == 64 || D == 128) {
+        // keys and values through LDS, one query tile a wave, the heads' rows of the table in LDS
+        if (g_attn_tune != 1 && a.page_shift >= 4 && a.page_size >= 512 / D && a.bias_len <= ATTN_BIAS_LDS) {
+          const dim3 lgrid((max_q_len + 15) / 16, kv_groups, n_req);
+          hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 1, 3, 3, true>), lgrid, dim3(256), 0, s, a, skip);
+          return 0;
+        }
+      }
       const dim3 grid((max_q_len + rows - 1) / rows, kv_groups, n_req);
       if (two)
         hipLaunchKernelGGL((attn_prefill_kernel<D, 2, true>), grid, dim3(256), 0, s, a, skip);
