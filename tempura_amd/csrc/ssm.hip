@@ -83,10 +83,11 @@ extern "C" int tp_causal_conv(const float* in, int in_stride, int col0, const fl
 // xbc [n, channels] float32 holds, per token, x [heads * head_dim] | B [groups * state] | C [groups * state] (after
 // the convolution); dt_raw is column dt_col0 + h of the projection's rows.
 //
-// A block owns one request, one head and PC = 256 / R value columns; R lanes (a power of two, neighbours in a
-// wave) share a column and split the state index among them, NPT consecutive entries each, in registers.
+// A block owns one request, one head and PC = (256 / R) * TP value columns; a thread holds TN consecutive state
+// entries of TP neighbouring columns in registers, and the R lanes (a power of two, neighbours in a wave) that share
+// those columns split the state index among them.
 // Tokens are taken TC at a time: their B, C, x, dt and decay are staged in LDS by all threads (rows padded with
-// zeros to R * NPT entries, so the run itself needs no bounds), then the run over the chunk is register
+// zeros to R * TN entries, so the run itself needs no bounds), then the run over the chunk is register
 // arithmetic, 16-byte LDS reads that most lanes share, and one reduction over the R lanes per token (row
 // permutes up to 16 lanes, which cost an instruction each and no trip through LDS).
 //
@@ -133,59 +134,69 @@ __device__ inline float lanes_sum(float v, int R) {
   return v;
 }
 
-template <int NPT>
+template <int TN, int TP>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(ScanArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  const int N = a.n_state, P = a.head_dim, R = a.R, PC = 256 / a.R, TC = a.TC;
-  const int NS = R * NPT;          // padded row of B and C
+  const int N = a.n_state, P = a.head_dim, R = a.R, CG = 256 / a.R, PC = CG * TP, TC = a.TC;
+  const int NS = R * TN;           // padded row of B and C
   float* Bs = lds;                 // [TC, NS]
   float* Cs = Bs + (size_t)TC * NS;
   float* xs = Cs + (size_t)TC * NS; // [TC, PC]
   float* dts = xs + (size_t)TC * PC;
   float* das = dts + TC;
   const int r = blockIdx.x, h = blockIdx.y;
-  const int slice = blockIdx.z % ((P + PC - 1) / PC), pc = blockIdx.z / ((P + PC - 1) / PC);
-  const int col = threadIdx.x / R, rr = threadIdx.x % R;
-  const int p = slice * PC + col;
-  const bool active = p < P;
+  const int slices = (P + PC - 1) / PC;
+  const int slice = blockIdx.z % slices, pc = blockIdx.z / slices;
+  const int cg = threadIdx.x / R, rr = threadIdx.x % R;
+  const int p0 = slice * PC + cg * TP;      // this thread's first value column
   const int g = h / (a.heads / a.groups);
   const int run0 = a.cu_seqlens[r], run_len = a.cu_seqlens[r + 1] - run0;
   if (run_len <= 0) return;
   const int inner = a.heads * P;
-  const int n0 = rr * NPT;
+  const int n0 = rr * TN;
   float* S = a.state + (size_t)a.state_slots[r] * a.state_stride + a.state_off + (size_t)h * N * P;
   const int pieces = a.mode == SCAN_DIRECT ? 1 : (run_len + a.piece - 1) / a.piece;
   float* PS = a.piece_state + ((size_t)(r * a.heads + h) * a.max_pieces) * N * P;
   float* PD = a.piece_decay + (size_t)(r * a.heads + h) * a.max_pieces;
+#define SCAN_HAS(i, j) (n0 + (i) < N && p0 + (j) < P)
+#define SCAN_AT(i, j) ((size_t)(n0 + (i)) * P + p0 + (j))
 
   if (a.mode == SCAN_CARRY) {
     // the state each piece starts from, in place of what it ended with from zero; then the request's new state
-    float cur[NPT];
+    float cur[TN][TP];
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) cur[i] = (active && n0 + i < N) ? S[(size_t)(n0 + i) * P + p] : 0.f;
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TP; ++j) cur[i][j] = SCAN_HAS(i, j) ? S[SCAN_AT(i, j)] : 0.f;
     for (int c = 0; c < pieces; ++c) {
       const float decay = PD[c];
       float* ps = PS + (size_t)c * N * P;
 #pragma unroll
-      for (int i = 0; i < NPT; ++i)
-        if (active && n0 + i < N) {
-          const float local = ps[(size_t)(n0 + i) * P + p];
-          ps[(size_t)(n0 + i) * P + p] = cur[i];
-          cur[i] = fmaf(decay, cur[i], local);
-        }
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TP; ++j)
+          if (SCAN_HAS(i, j)) {
+            const float local = ps[SCAN_AT(i, j)];
+            ps[SCAN_AT(i, j)] = cur[i][j];
+            cur[i][j] = fmaf(decay, cur[i][j], local);
+          }
     }
 #pragma unroll
-    for (int i = 0; i < NPT; ++i)
-      if (active && n0 + i < N) S[(size_t)(n0 + i) * P + p] = cur[i];
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TP; ++j)
+        if (SCAN_HAS(i, j)) S[SCAN_AT(i, j)] = cur[i][j];
     return;
   }
   if (pc >= pieces) return;
   const int start = a.mode == SCAN_DIRECT ? run0 : run0 + pc * a.piece;
   const int len = a.mode == SCAN_DIRECT ? run_len : min(a.piece, run_len - pc * a.piece);
   const float* init = a.mode == SCAN_DIRECT ? S : (a.mode == SCAN_OUTPUT ? PS + (size_t)pc * N * P : nullptr);
-  float st[NPT];
+  float st[TN][TP];
 #pragma unroll
-  for (int i = 0; i < NPT; ++i) st[i] = (init != nullptr && active && n0 + i < N) ? init[(size_t)(n0 + i) * P + p] : 0.f;
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TP; ++j) st[i][j] = (init != nullptr && SCAN_HAS(i, j)) ? init[SCAN_AT(i, j)] : 0.f;
   const float A = -expf(a.a_log[h]);
   const float dtb = a.dt_bias[h], Dh = a.d_skip[h];
   const bool write_y = a.mode != SCAN_LOCAL;
@@ -219,44 +230,57 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(ScanArgs a) {
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
       const float dt = dts[tt], da = das[tt];
-      const float xv = xs[tt * PC + col];
-      const float dx = dt * xv;
+      float xv[TP], dx[TP], acc[TP];
+#pragma unroll
+      for (int j = 0; j < TP; ++j) {
+        xv[j] = xs[tt * PC + cg * TP + j];
+        dx[j] = dt * xv[j];
+        acc[j] = 0.f;
+      }
       const float* Bt = Bs + (size_t)tt * NS + n0;
       const float* Ct = Cs + (size_t)tt * NS + n0;
-      float bv[NPT], cv[NPT];
-      if constexpr (NPT % 4 == 0) {
+      float bv[TN], cv[TN];
+      if constexpr (TN % 4 == 0) {
 #pragma unroll
-        for (int i = 0; i < NPT; i += 4) {
+        for (int i = 0; i < TN; i += 4) {
           const float4 b4 = *(const float4*)(Bt + i), c4 = *(const float4*)(Ct + i);
           bv[i] = b4.x; bv[i + 1] = b4.y; bv[i + 2] = b4.z; bv[i + 3] = b4.w;
           cv[i] = c4.x; cv[i + 1] = c4.y; cv[i + 2] = c4.z; cv[i + 3] = c4.w;
         }
       } else {
 #pragma unroll
-        for (int i = 0; i < NPT; ++i) {
+        for (int i = 0; i < TN; ++i) {
           bv[i] = Bt[i];
           cv[i] = Ct[i];
         }
       }
-      float acc = 0.f;
 #pragma unroll
-      for (int i = 0; i < NPT; ++i) {
-        st[i] = fmaf(da, st[i], dx * bv[i]);
-        acc = fmaf(st[i], cv[i], acc);
-      }
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TP; ++j) {
+          st[i][j] = fmaf(da, st[i][j], dx[j] * bv[i]);
+          acc[j] = fmaf(st[i][j], cv[i], acc[j]);
+        }
       dt_sum += dt;
       if (write_y) {
-        acc = lanes_sum(acc, R);
-        if (rr == 0 && active) a.y[(size_t)(start + t0 + tt) * inner + h * P + p] = fmaf(Dh, xv, acc);
+#pragma unroll
+        for (int j = 0; j < TP; ++j) {
+          const float total = lanes_sum(acc[j], R);
+          if (rr == 0 && p0 + j < P) a.y[(size_t)(start + t0 + tt) * inner + h * P + p0 + j] = fmaf(Dh, xv[j], total);
+        }
       }
     }
   }
   if (a.mode == SCAN_OUTPUT) return;
   float* dst = a.mode == SCAN_DIRECT ? S : PS + (size_t)pc * N * P;
 #pragma unroll
-  for (int i = 0; i < NPT; ++i)
-    if (active && n0 + i < N) dst[(size_t)(n0 + i) * P + p] = st[i];
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TP; ++j)
+      if (SCAN_HAS(i, j)) dst[SCAN_AT(i, j)] = st[i][j];
   if (a.mode == SCAN_LOCAL && slice == 0 && threadIdx.x == 0) PD[pc] = expf(A * dt_sum);
+#undef SCAN_HAS
+#undef SCAN_AT
 }
 
 // scratch floats a scan of n_req requests whose longest run has max_run tokens needs (0: it runs in one launch)
@@ -288,19 +312,23 @@ extern "C" int tp_ssm_scan(const float* xbc, const float* proj, int proj_stride,
   a.cu_seqlens = cu_seqlens; a.state_slots = state_slots; a.y = y;
   a.heads = heads; a.head_dim = head_dim; a.n_state = n_state; a.groups = groups;
   a.channels = heads * head_dim + 2 * groups * n_state;
-  // lanes per column: enough that a lane holds at most 32 state entries, and no more columns than the head has
-  // values.  Few lanes a column and many entries a lane: the B and C rows a block stages serve more columns, and
-  // more of a wave's instructions are the recurrence's own.
+  // A thread holds TN state entries of TP value columns; the R lanes that share those columns split the state index.
+  // Two columns a thread halve what a token's B and C cost in LDS reads for each update of the state; sixteen
+  // entries a lane keep most of a wave's instructions the recurrence's own.  No more columns a block than the head has.
+  const int TP = (head_dim >= 2 && n_state <= 1024) ? 2 : 1;
+  const int cap = TP == 2 ? 16 : 32;
   int R = 1;
-  while (R < 64 && R * 32 < n_state) R *= 2;
+  while (R < 64 && R * cap < n_state) R *= 2;
   int pc_pow2 = 1;
   while (pc_pow2 < head_dim) pc_pow2 *= 2;
-  while (R < 64 && 256 / R > pc_pow2) R *= 2;
+  while (R < 64 && (256 / R) * TP > pc_pow2) R *= 2;
   const int per_lane = (n_state + R - 1) / R;
-  const int npt = per_lane <= 1 ? 1 : (per_lane <= 2 ? 2 : (per_lane <= 4 ? 4 : (per_lane <= 8 ? 8 : (per_lane <= 16 ? 16 : 32))));
+  int tn = 1;
+  while (tn < per_lane) tn *= 2;
+  TP_REQUIRE(tn <= cap, "ssm_scan: state size %d does not fit a block", n_state);
   a.R = R;
-  const int PC = 256 / R;
-  const int per_token = 2 * R * npt + PC + 2;
+  const int PC = (256 / R) * TP;
+  const int per_token = 2 * R * tn + PC + 2;
   int TC = (32 * 1024 / 4) / per_token;
   TC = TC < 1 ? 1 : (TC > 64 ? 64 : TC);
   a.TC = TC;
@@ -314,15 +342,23 @@ extern "C" int tp_ssm_scan(const float* xbc, const float* proj, int proj_stride,
   a.piece_decay = scratch ? scratch + (size_t)n_req * heads * a.max_pieces * n_state * head_dim : nullptr;
   TP_REQUIRE(piece == 0 || (scratch != nullptr && scratch_floats >= need), "ssm_scan: scratch of %zu floats needed", need);
   TP_REQUIRE((long)slices * a.max_pieces <= 65535, "ssm_scan: too many pieces");
-#define SCAN_LAUNCH(NPT, GRID) hipLaunchKernelGGL(ssm_scan_kernel<NPT>, GRID, dim3(256), shmem, s, a)
-#define SCAN_DISPATCH(GRID)            \
-  do {                                 \
-    if (npt == 1) SCAN_LAUNCH(1, GRID);      \
-    else if (npt == 2) SCAN_LAUNCH(2, GRID); \
-    else if (npt == 4) SCAN_LAUNCH(4, GRID); \
-    else if (npt == 8) SCAN_LAUNCH(8, GRID); \
-    else if (npt == 16) SCAN_LAUNCH(16, GRID); \
-    else SCAN_LAUNCH(32, GRID);              \
+#define SCAN_LAUNCH(TN_, TP_, GRID) hipLaunchKernelGGL((ssm_scan_kernel<TN_, TP_>), GRID, dim3(256), shmem, s, a)
+#define SCAN_DISPATCH(GRID)                                \
+  do {                                                     \
+    if (TP == 2) {                                         \
+      if (tn == 1) SCAN_LAUNCH(1, 2, GRID);                \
+      else if (tn == 2) SCAN_LAUNCH(2, 2, GRID);           \
+      else if (tn == 4) SCAN_LAUNCH(4, 2, GRID);           \
+      else if (tn == 8) SCAN_LAUNCH(8, 2, GRID);           \
+      else SCAN_LAUNCH(16, 2, GRID);                       \
+    } else {                                               \
+      if (tn == 1) SCAN_LAUNCH(1, 1, GRID);                \
+      else if (tn == 2) SCAN_LAUNCH(2, 1, GRID);           \
+      else if (tn == 4) SCAN_LAUNCH(4, 1, GRID);           \
+      else if (tn == 8) SCAN_LAUNCH(8, 1, GRID);           \
+      else if (tn == 16) SCAN_LAUNCH(16, 1, GRID);         \
+      else SCAN_LAUNCH(32, 1, GRID);                       \
+    }                                                      \
   } while (0)
   if (piece == 0) {
     a.mode = SCAN_DIRECT;
