@@ -69,6 +69,13 @@ __device__ inline void rope_cos_sin(int pos, double inv_freq, float factor, floa
 // rotates what it holds and stores q as bfloat16 [M, heads, head_dim], k into the cache place slots[m] and v
 // into the transposed value cache: the rotation and cache-write kernel between the projection and the
 // attention is gone.  The arithmetic is that kernel's, on the same float32 sums.
+// The activation of a gated product's epilogue: with g' = min(g, limit) and u' = clamp(u, -limit, limit) when
+// limit > 0, the result is g' * sigmoid((1 + extra_slope) * g') * (u' + offset).  All zero is the gated SiLU
+// (SwiGLU), bit for bit as without these constants; a kernel gets them by value.
+struct GateAct {
+  float extra_slope, limit, offset;
+};
+
 struct RopeOut {
   const int* positions;      // [M]
   const int* slots;          // [M] cache place (page * page_size + offset)
@@ -80,8 +87,19 @@ struct RopeOut {
   bf16_t* q_out;
   bf16_t* k_cache;           // [page, kv_head, page_size, head_dim]
   bf16_t* v_cache;           // [page, kv_head, head_dim, page_size]
+  GateAct gate;              // (mode OUT_SWIGLU of the same kernels: the activation's constants)
 };
 enum { OUT_ROPE = 4 };
+
+// g * sigmoid(slope g) * (u + offset) with the hardware's exp2 and reciprocal (one ulp each; the result is rounded to
+// bfloat16), the same arithmetic in every bfloat16 product, whatever the number of rows
+__device__ inline float gate_mul(float g, float u, const GateAct& a) {
+  if (a.limit > 0.f) {
+    g = fminf(g, a.limit);
+    u = fminf(fmaxf(u, -a.limit), a.limit);
+  }
+  return g * (u + a.offset) * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * (-1.4426950408889634f * (1.0f + a.extra_slope))));
+}
 
 __device__ inline float wave_sum(float v) {
 #pragma unroll

@@ -144,7 +144,7 @@ static void launch_generic(const void* x, const void* w, void* out, int M, int N
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
                    float* scratch, size_t scratch_floats, const float* pre_ss, int pre_count, float pre_eps,
                    const void* post_w, void* post_xg, float* post_ss, int layout, int defer_reduce, int* splits_out,
-                   hipStream_t s);
+                   GateAct gate, hipStream_t s);
 
 int tp_linear_rope_mfma(const void* x, const void* w, int w_tiled, int M, int N, int K, const float* pre_ss, int pre_count,
                         float pre_eps, const int* positions, const int* slots, const double* inv_freq, int rotary_dim,
@@ -193,7 +193,8 @@ extern "C" int tp_linear_rope(const void* x, const void* w, int w_tiled, int M, 
 extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
                                int N, int K, int allow_mfma, float* scratch, size_t scratch_floats,
                                const float* pre_ss, int pre_count, float pre_eps, const void* post_w, void* post_xg,
-                               float* post_ss, int layout, int defer_reduce, int* splits_out, hipStream_t s) {
+                               float* post_ss, int layout, int defer_reduce, int* splits_out, float gate_slope,
+                               float gate_limit, float gate_offset, hipStream_t s) {
   if (splits_out) *splits_out = 1;
   TP_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   TP_REQUIRE(accumulate != 1 || out_dt == TP_F32, "linear: accumulating output must be float32");
@@ -211,8 +212,10 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
   }
   if (accumulate == 2) {  // gated-SiLU epilogue: only the matrix-core kernels have it
     TP_REQUIRE(in_dt == TP_BF16 && allow_mfma, "linear: the gated epilogue needs bfloat16 operands");
+    // (the epilogue's activation: slope of the sigmoid, limit of both branches (<= 0: none), what is added to the up branch)
+    const GateAct gate = {gate_slope - 1.0f, gate_limit > 0.f ? gate_limit : 0.f, gate_offset};
     const int r = tp_linear_mfma(x, w, out, out_dt, 2, M, N, K, scratch, scratch_floats, pre_ss, pre_count, pre_eps,
-                                 nullptr, nullptr, nullptr, layout, 0, nullptr, s);
+                                 nullptr, nullptr, nullptr, layout, 0, nullptr, gate, s);
     TP_REQUIRE(r >= 0, "linear: sizes M=%d N=%d K=%d do not fit the gated epilogue", M, N, K);
     return r;
   }
@@ -220,7 +223,7 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
   if (M == 0) return 0;
   if (in_dt == TP_BF16 && allow_mfma) {
     const int r = tp_linear_mfma(x, w, out, out_dt, accumulate, M, N, K, scratch, scratch_floats, pre_ss, pre_count,
-                                 pre_eps, post_w, post_xg, post_ss, layout, defer_reduce, splits_out, s);
+                                 pre_eps, post_w, post_xg, post_ss, layout, defer_reduce, splits_out, GateAct{}, s);
     if (r >= 0) return r;
   }
   TP_REQUIRE(!(layout & 4), "linear: no kernel for tiled weights at M=%d N=%d K=%d", M, N, K);

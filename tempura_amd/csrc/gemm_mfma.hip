@@ -25,11 +25,6 @@ typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 // 8*b + i is silu(row 16*b + i) * (row 16*b + 8 + i), stored as bfloat16 [M, N / 2].
 enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_ACC_F32 = 2, OUT_SWIGLU = 3 };
 
-// g * sigmoid(g) * u with the hardware's exp2 and reciprocal (one ulp each; the result is rounded to bfloat16),
-// the same arithmetic in every bfloat16 product, whatever the number of rows
-__device__ inline float silu_mul(float g, float u) {
-  return g * u * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
-}
 
 __device__ inline bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
 
@@ -252,7 +247,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
 #pragma unroll
         for (int i = 0; i < WAVES; ++i) u += red[i][jt][q + 128];
         if (MT == 1) u *= rstd[l & 15];
-        store_gated(out, layout, M, N / 2, m, (n0 + j * 16) / 2 + (l >> 4) * 4 + r, silu_mul(v, u));
+        store_gated(out, layout, M, N / 2, m, (n0 + j * 16) / 2 + (l >> 4) * 4 + r, gate_mul(v, u, rp.gate));
       }
     } else if (MT == 1 && post.w != nullptr) {
       // residual add, and the next norm's preparation (mode is OUT_ACC_F32)
@@ -409,7 +404,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const bf16_
 #pragma unroll
         for (int i = 0; i < WAVES; ++i) u += red[ge * WAVES + i][j][q + 128];
         u *= rstd[m];
-        store_gated(out, layout, M, N / 2, m, nt0 / 2 + (l >> 4) * 4 + r, silu_mul(v, u));
+        store_gated(out, layout, M, N / 2, m, nt0 / 2 + (l >> 4) * 4 + r, gate_mul(v, u, rp.gate));
       }
     } else if (post.w != nullptr) {
       float sq = 0.f;
@@ -455,7 +450,7 @@ template <int BK, int WMT, int WNT>
 __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(const bf16_t* __restrict__ x,
                                                               const bf16_t* __restrict__ w, void* __restrict__ out,
                                                               float* __restrict__ partial, int mode, int M, int N,
-                                                              int K, int xcd_order) {
+                                                              int K, int xcd_order, GateAct ga) {
   constexpr int BM = 32 * WMT, BN = 32 * WNT;
   constexpr int LD = BK + 8;            // padded row, in bf16 elements (conflict-free 16-byte reads)
   constexpr int CPR = BK / 8;           // 16-byte chunks per tile row
@@ -557,7 +552,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(const bf16_t* __re
         } else if (mode == OUT_SWIGLU) {
           const float u = __shfl_xor(acc[i][j][r], 8, 64);   // the up row sits eight columns to the right
           if ((lane & 8) == 0 && n + 8 < N)
-            ((bf16_t*)out)[(size_t)m * (N / 2) + nt / 2 + (lane & 7)] = float_to_bf16(silu_mul(acc[i][j][r], u));
+            ((bf16_t*)out)[(size_t)m * (N / 2) + nt / 2 + (lane & 7)] = float_to_bf16(gate_mul(acc[i][j][r], u, ga));
         } else if (n < N) {
           store_out(out, mode, (size_t)m * N + n, acc[i][j][r]);
         }
@@ -568,7 +563,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(const bf16_t* __re
 
 // Adds the K splits of `partial` [splits, M, N] in ascending order and applies the epilogue.
 __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ out, int mode,
-                                          int splits, int M, int N) {
+                                          int splits, int M, int N, GateAct ga) {
   const size_t total = (size_t)M * N;
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (mode == OUT_SWIGLU) {
@@ -582,7 +577,7 @@ __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, voi
       g += partial[(size_t)s * total + (size_t)m * N + ng];
       u += partial[(size_t)s * total + (size_t)m * N + ng + 8];
     }
-    ((bf16_t*)out)[idx] = float_to_bf16(silu_mul(g, u));
+    ((bf16_t*)out)[idx] = float_to_bf16(gate_mul(g, u, ga));
     return;
   }
   if (idx >= total) return;
@@ -662,10 +657,11 @@ static int g_tune_order = 0;   // large products: 1 tiled kernel, plain block or
 
 // Defined in gemm_pipe.hip; 0 when it took the product, -1 when the sizes are not its own.
 int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
-                   size_t scratch_floats, int tune_splits, const RopeOut* rope, int defer, int* splits_out, hipStream_t s);
+                   size_t scratch_floats, int tune_splits, const RopeOut* rope, int defer, int* splits_out, GateAct gate,
+                   hipStream_t s);
 
 int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
-                     size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s);
+                     size_t scratch_floats, int tune_splits, int defer, int* splits_out, GateAct gate, hipStream_t s);
 
 extern int g_pipe_big;
 // order: 1 tiled plain, 2 tiled XCD-aware, 3 pipelined; 5 / 6: pipelined with 256 x 256 tiles always / never;
@@ -789,7 +785,7 @@ int tp_linear_rope_mfma(const void* x, const void* w, int w_tiled, int M, int N,
     // multiple of 64; the wider tiles are left out unless the heads are multiples of 128), with the step's table
     // of cosines and sines
     if (head_dim % 64 != 0 || rotary_dim % 8 != 0 || cos_sin == nullptr || pre_ss != nullptr || page_size % 8 != 0) return -1;
-    return tp_linear_pipe((const bf16_t*)x, (const bf16_t*)w, w_tiled & 1, nullptr, OUT_ROPE, M, N, K, nullptr, 0, 0, &rp, 0, nullptr, s);
+    return tp_linear_pipe((const bf16_t*)x, (const bf16_t*)w, w_tiled & 1, nullptr, OUT_ROPE, M, N, K, nullptr, 0, 0, &rp, 0, nullptr, GateAct{}, s);
   }
   launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, (w_tiled & 1 ? W_TILED : 0) | (w_tiled & 2 ? X_KBLOCKED : 0),
                    pre, post, rp, s);
@@ -801,7 +797,7 @@ int tp_linear_rope_mfma(const void* x, const void* w, int w_tiled, int M, int N,
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
                    float* scratch, size_t scratch_floats, const float* pre_ss, int pre_count, float pre_eps,
                    const void* post_w, void* post_xg, float* post_ss, int layout, int defer_reduce, int* splits_out,
-                   hipStream_t s) {
+                   GateAct gate, hipStream_t s) {
   if (splits_out) *splits_out = 1;
   if (K % 32 != 0) return -1;
   const int w_tiled = (layout & W_TILED) != 0;
@@ -819,7 +815,8 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
   const bf16_t* xb = (const bf16_t*)x;
   const bf16_t* wb = (const bf16_t*)w;
   const bool mid_ok = scratch != nullptr && g_tune_mid != 1;
-  const RopeOut no_rope = {};
+  RopeOut no_rope = {};
+  no_rope.gate = gate;      // (the kernels read the gated epilogue's constants from here)
   if (M <= 16 || (M <= 64 && !mid_ok)) {
     if (M <= 16)
       launch_skinny<1>(xb, wb, out, mode, M, N, K, layout, pre, post, no_rope, s);
@@ -837,10 +834,10 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
     const bool pipe = g_tune_order ? g_tune_order == 3 : M > 64;
     const bool pipe64 = !pipe && M <= 128 && scratch != nullptr && g_tune_mid != 2;
     if (pipe && tp_linear_pipe(xb, wb, w_tiled, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, nullptr, defer_reduce,
-                               splits_out, s) == 0) {
+                               splits_out, gate, s) == 0) {
       // taken by the pipelined kernel
     } else if (pipe64 && tp_linear_pipe64(xb, wb, w_tiled, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits,
-                                          defer_reduce, splits_out, s) == 0) {
+                                          defer_reduce, splits_out, gate, s) == 0) {
       // taken by the 64-row pipelined kernel
     } else if (w_tiled) {
       return -1;   // the kernels below read row-major weights only
@@ -854,10 +851,10 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
       }
       if (K % 64 == 0)
         hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64, 4, 4>), grid, dim3(256), 0, s, xb, wb, out, nullptr, mode, M, N, K,
-                           xcd_order);
+                           xcd_order, gate);
       else
         hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32, 4, 4>), grid, dim3(256), 0, s, xb, wb, out, nullptr, mode, M, N, K,
-                           xcd_order);
+                           xcd_order, gate);
     } else {
       const int nb = (N + 127) / 128, mb = (M + 63) / 64;
       int splits = g_tune_splits ? g_tune_splits : (512 + nb * mb - 1) / (nb * mb);
@@ -866,15 +863,15 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
       while (splits > 1 && (size_t)splits * M * N > scratch_floats) --splits;
       const dim3 grid(nb, mb, splits);
       if (K % 64 == 0)
-        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K, 0);
+        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K, 0, gate);
       else
-        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K, 0);
+        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K, 0, gate);
       if (splits > 1 && defer_reduce && splits_out != nullptr && mode != OUT_SWIGLU) {
         *splits_out = splits;   // the caller's next kernel adds the partial sums [splits, M, N] in `scratch`
       } else if (splits > 1) {
         const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
         hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out,
-                           mode, splits, M, N);
+                           mode, splits, M, N, gate);
       }
     }
   }

@@ -50,10 +50,6 @@ constexpr int LPW = 12;        // direct loads per wave and stage: eight of x ro
 constexpr int CLD = 64 + 4;    // padded row of a wave's result tile in LDS, in floats
 
 __device__ inline bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
-// g * sigmoid(g) * u with the hardware's exp2 and reciprocal (one ulp each; the result is rounded to bfloat16)
-__device__ inline float silu_mul(float g, float u) {
-  return g * u * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
-}
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 // two floats to two bfloat16 (round to nearest even) in one instruction
@@ -173,7 +169,8 @@ __device__ inline void half_step(f32x4_t (&acc)[8][4], const Frags& cur, Frags& 
 // multiply for the address, a row check and a branch took as long as the store itself, and stores of 8 bytes
 // per lane twice as long as stores of 16.)
 template <int ROWS, int COLS, int LD>
-__device__ inline void emit_tile_fast(const float* ct, int lane, int mrow0, int ncol0, void* out, int mode, int ldo) {
+__device__ inline void emit_tile_fast(const float* ct, int lane, int mrow0, int ncol0, void* out, int mode, int ldo,
+                                      const GateAct& ga) {
   if (mode == OUT_SWIGLU) {
     // eight outputs per lane: the eight gate columns of a group of sixteen and the eight up columns after them
     constexpr int LPR = COLS / 16, RPP = 64 / LPR, PASSES = ROWS / RPP, B = PASSES < 4 ? PASSES : 4;
@@ -195,10 +192,10 @@ __device__ inline void emit_tile_fast(const float* ct, int lane, int mrow0, int 
 #pragma unroll
       for (int u = 0; u < B; ++u) {
         u32x4_t pk;
-        pk[0] = pack_bf16(silu_mul(g0[u][0], u0[u][0]), silu_mul(g0[u][1], u0[u][1]));
-        pk[1] = pack_bf16(silu_mul(g0[u][2], u0[u][2]), silu_mul(g0[u][3], u0[u][3]));
-        pk[2] = pack_bf16(silu_mul(g1[u][0], u1[u][0]), silu_mul(g1[u][1], u1[u][1]));
-        pk[3] = pack_bf16(silu_mul(g1[u][2], u1[u][2]), silu_mul(g1[u][3], u1[u][3]));
+        pk[0] = pack_bf16(gate_mul(g0[u][0], u0[u][0], ga), gate_mul(g0[u][1], u0[u][1], ga));
+        pk[1] = pack_bf16(gate_mul(g0[u][2], u0[u][2], ga), gate_mul(g0[u][3], u0[u][3], ga));
+        pk[2] = pack_bf16(gate_mul(g1[u][0], u1[u][0], ga), gate_mul(g1[u][1], u1[u][1], ga));
+        pk[3] = pack_bf16(gate_mul(g1[u][2], u1[u][2], ga), gate_mul(g1[u][3], u1[u][3], ga));
         *(u32x4_t*)(dst + (p0 + u) * step) = pk;
       }
     }
@@ -414,9 +411,10 @@ __device__ inline void emit_tile_rope(const float* ct, int lane, int mrow0, int 
 // columns ncol0.. of the launch's N (row stride ldo).  Four rows are read from LDS before the first of them is
 // stored, so that the reads (and, when adding into `out`, the loads) overlap.
 template <int ROWS, int COLS, int LD>
-__device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0, void* out, int mode, int M, int N, int ldo) {
+__device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0, void* out, int mode, int M, int N, int ldo,
+                                 const GateAct& ga) {
   if (mrow0 + ROWS <= M && ncol0 + COLS <= N && ldo % 8 == 0 && ((uintptr_t)out & 15) == 0) {
-    emit_tile_fast<ROWS, COLS, LD>(ct, lane, mrow0, ncol0, out, mode, ldo);
+    emit_tile_fast<ROWS, COLS, LD>(ct, lane, mrow0, ncol0, out, mode, ldo, ga);
     return;
   }
   if (mode == OUT_SWIGLU) {
@@ -440,8 +438,8 @@ __device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0
       for (int u = 0; u < B; ++u) {
         const int m = mrow0 + (p0 + u) * RPP + rr;
         u32x2_t pk;
-        pk[0] = pack_bf16(silu_mul(gt[u][0], up[u][0]), silu_mul(gt[u][1], up[u][1]));
-        pk[1] = pack_bf16(silu_mul(gt[u][2], up[u][2]), silu_mul(gt[u][3], up[u][3]));
+        pk[0] = pack_bf16(gate_mul(gt[u][0], up[u][0], ga), gate_mul(gt[u][1], up[u][1], ga));
+        pk[1] = pack_bf16(gate_mul(gt[u][2], up[u][2], ga), gate_mul(gt[u][3], up[u][3], ga));
         if (m < M) *(u32x2_t*)(ob + (size_t)m * ldo + ncol0 / 2 + o) = pk;
       }
     }
@@ -645,7 +643,7 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
     rope_fetch(fetched, lane, m0 + wm * 128 + 64, n0 + wn * 64, rp, M);
     emit_tile_rope<64, 64, CLD>(ct + 64 * CLD, lane, m0 + wm * 128 + 64, n0 + wn * 64, rp, M, fetched);
   } else {
-    emit_tile<128, 64, CLD>(ct, lane, m0 + wm * 128, n0 + wn * 64, out, mode, M, N, ldo);
+    emit_tile<128, 64, CLD>(ct, lane, m0 + wm * 128, n0 + wn * 64, out, mode, M, N, ldo, rp.gate);
   }
 }
 
@@ -898,7 +896,7 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
     if (mode == OUT_ROPE)                                                                                       \
       emit_tile_rope<32, 128, CLDB>(ct, lane, mw + (Q) * 32, nw, rp, M, fetched);                               \
     else                                                                                                        \
-      emit_tile<32, 128, CLDB>(ct, lane, mw + (Q) * 32, nw, out, mode, M, N, ldo);                              \
+      emit_tile<32, 128, CLDB>(ct, lane, mw + (Q) * 32, nw, out, mode, M, N, ldo, rp.gate);                             \
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                          \
   }
   QUARTER(0)
@@ -922,7 +920,7 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
     if (mode == OUT_ROPE)                                                                                       \
       emit_tile_rope<128, 32, CLDS>(ct, lane, mw, nw + (JB) * 16, rp, M, fetched);                              \
     else                                                                                                        \
-      emit_tile<128, 32, CLDS>(ct, lane, mw, nw + (JB) * 16, out, mode, M, N, ldo);                             \
+      emit_tile<128, 32, CLDS>(ct, lane, mw, nw + (JB) * 16, out, mode, M, N, ldo, rp.gate);                            \
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                          \
   }
 #define STRIP64(JB, H)                                                                                          \
@@ -935,7 +933,7 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
     if (mode == OUT_ROPE)                                                                                       \
       emit_tile_rope<64, 64, CLD>(ct, lane, mw + (H) * 64, nw + (JB) * 16, rp, M, fetched);                     \
     else                                                                                                        \
-      emit_tile<64, 64, CLD>(ct, lane, mw + (H) * 64, nw + (JB) * 16, out, mode, M, N, ldo);                    \
+      emit_tile<64, 64, CLD>(ct, lane, mw + (H) * 64, nw + (JB) * 16, out, mode, M, N, ldo, rp.gate);                   \
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                          \
   }
   static_assert(128 * CLDS >= 64 * CLD, "room for either strip");
@@ -1021,7 +1019,7 @@ __device__ inline void half_step64(f32x4_t (&acc)[2][NJ], const Frags64<NJ>& cur
 template <int NJ>
 __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                              void* __restrict__ out, float* __restrict__ partial,
-                                                             int mode, int M, int N, int K, int wt) {
+                                                             int mode, int M, int N, int K, int wt, GateAct ga) {
   constexpr int BNT = 32 * NJ, STAGE = (BM64 + BNT) * ROWB, LPWT = 2 + NJ;
   __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1131,7 +1129,7 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __res
 #pragma unroll
       for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLD + j * 16 + c] = acc[i][j][r];
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  emit_tile<32, 16 * NJ, CLD>(ct, lane, m0 + wm * 32, n0 + wn * 16 * NJ, out, mode, M, N, mode == OUT_SWIGLU ? N / 2 : N);
+  emit_tile<32, 16 * NJ, CLD>(ct, lane, m0 + wm * 32, n0 + wn * 16 * NJ, out, mode, M, N, mode == OUT_SWIGLU ? N / 2 : N, ga);
 }
 
 // ---- the same pipeline on 128 x 128 blocks ------------------------------------------------------------
@@ -1325,12 +1323,12 @@ __global__ __launch_bounds__(256) void gemm_pipe128_kernel(const bf16_t* __restr
   if (mode == OUT_ROPE)
     emit_tile_rope<64, 64, CLD>(ct, lane, mw, nw, rp, M, fetched);
   else
-    emit_tile<64, 64, CLD>(ct, lane, mw, nw, out, mode, M, N, ldo);
+    emit_tile<64, 64, CLD>(ct, lane, mw, nw, out, mode, M, N, ldo, rp.gate);
 }
 
 // Defined in gemm_mfma.hip.
 __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ out, int mode,
-                                          int splits, int M, int N);
+                                          int splits, int M, int N, GateAct ga);
 
 int g_pipe_mid = 0;   // tuning: 1 = 128 x 128 blocks for every product of more than 128 rows, 2 = never
 
@@ -1390,12 +1388,13 @@ static int splits256(long tiles, int KT, int M, int N, const float* scratch, siz
 // The 128 x 128 blocks.  Returns 0 when launched.
 static int tp_linear_pipe128(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K,
                              float* scratch, size_t scratch_floats, const RopeOut* rope, int defer, int* splits_out,
-                             hipStream_t s) {
+                             GateAct gate, hipStream_t s) {
   const int MB = (M + BM128 - 1) / BM128, NB = (N + BN128 - 1) / BN128;
   const long tiles = (long)MB * NB;
   const int splits = splits128(M, N, K, scratch != nullptr && rope == nullptr, scratch_floats);
   RopeOut rp = {};
   if (rope != nullptr) rp = *rope;
+  rp.gate = gate;
   const int ldo = mode == OUT_SWIGLU ? N / 2 : N;
   const long per_xcd = (tiles * splits + 7) / 8;
   if (8 * per_xcd > 0x7fffffffL) return -1;
@@ -1406,7 +1405,7 @@ static int tp_linear_pipe128(const bf16_t* x, const bf16_t* w, int w_tiled, void
   } else if (splits > 1) {
     const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,
-                       splits, M, N);
+                       splits, M, N, gate);
   }
   return 0;
 }
@@ -1415,7 +1414,8 @@ static int tp_linear_pipe128(const bf16_t* x, const bf16_t* w, int w_tiled, void
 // float32 partial sums: with few result tiles K is split over blocks until there is work for every CU.
 int g_pipe_big = 0;   // tuning: 1 = 256 x 256 tiles for every whole block of 256 columns, 2 = never; 3 = 256 x 192 wherever N allows, 4 = never
 int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
-                   size_t scratch_floats, int tune_splits, const RopeOut* rope, int defer, int* splits_out, hipStream_t s) {
+                   size_t scratch_floats, int tune_splits, const RopeOut* rope, int defer, int* splits_out, GateAct gate,
+                   hipStream_t s) {
   if ((mode == OUT_ROPE) != (rope != nullptr)) return -1;
   if (w_tiled && N % 16 != 0) return -1;
   if (K % BK != 0 || K < BK) return -1;
@@ -1434,7 +1434,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
     mid = pipe_cost(tiles128 * s128, (KT + s128 - 1) / s128, STEP128_US, s128, M, N) <
           pipe_cost(tiles * s256, (KT + s256 - 1) / s256, STEP256_US, s256, M, N);
   }
-  if (mid) return tp_linear_pipe128(x, w, w_tiled, out, mode, M, N, K, scratch, scratch_floats, rope, defer, splits_out, s);
+  if (mid) return tp_linear_pipe128(x, w, w_tiled, out, mode, M, N, K, scratch, scratch_floats, rope, defer, splits_out, gate, s);
   // (see tile_of_block) strips of at most eight row blocks, all about as tall; a launch of nb column blocks has
   // 8 x ceil(MB x nb / 8) blocks
   const int strips = (MB + 7) / 8;
@@ -1447,6 +1447,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
   const int ldo = mode == OUT_SWIGLU ? N / 2 : N;
   RopeOut rp = {};
   if (rope != nullptr) rp = *rope;
+  rp.gate = gate;
   // Whole rounds of 256 x 256 tiles first (see gemm_pipe_big_kernel), the columns that are left as above.
   // How many blocks of 256 columns take the big tiles: all, none, or whole rounds of 256 tiles, whichever
   // needs the fewest rounds when a big tile is priced at 1.72 small ones (measured: 113 against 65 us at
@@ -1506,7 +1507,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
   } else if (splits > 1) {
     const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,
-                       splits, M, N);
+                       splits, M, N, gate);
   }
   return 0;
 }
@@ -1515,7 +1516,7 @@ int g_pipe64_narrow = 0;   // tuning: 1 = blocks of 64 columns always, 2 = never
 // The 64-row pipeline (17..64 rows; up to 128 where the other kernels do not take the sizes).  `defer`: when K is split, leave the partial sums in `scratch` for the
 // caller's next kernel and report their number through *splits_out.
 int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
-                     size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s) {
+                     size_t scratch_floats, int tune_splits, int defer, int* splits_out, GateAct gate, hipStream_t s) {
   if (K % BK != 0 || K < BK || M > 128) return -1;
   if (w_tiled && N % 16 != 0) return -1;
   if ((size_t)(BM64 - 1) * K * 2 + 128 >= ((size_t)1 << 31)) return -1;
@@ -1554,16 +1555,16 @@ int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, i
   const bool leave = defer && splits > 1 && splits_out != nullptr && mode != OUT_SWIGLU;
   if (narrow)
     hipLaunchKernelGGL(gemm_pipe64_kernel<2>, dim3((unsigned)tiles, splits), dim3(256), 0, s, x, w, out,
-                       splits > 1 ? scratch : nullptr, mode, M, N, K, w_tiled);
+                       splits > 1 ? scratch : nullptr, mode, M, N, K, w_tiled, gate);
   else
     hipLaunchKernelGGL(gemm_pipe64_kernel<4>, dim3((unsigned)tiles, splits), dim3(256), 0, s, x, w, out,
-                       splits > 1 ? scratch : nullptr, mode, M, N, K, w_tiled);
+                       splits > 1 ? scratch : nullptr, mode, M, N, K, w_tiled, gate);
   if (leave) {
     *splits_out = splits;
   } else if (splits > 1) {
     const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,
-                       splits, M, N);
+                       splits, M, N, gate);
   }
   return 0;
 }

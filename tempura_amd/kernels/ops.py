@@ -538,11 +538,15 @@ def _pre_args(x):
     return x, (_ptr(None), 0, ctypes.c_float(0.0)), (tuple(x.shape) if x.dim() == 2 else None), 0
 
 
-def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
+def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False, slope: float = 1.0, limit: float = 0.0, up_offset: float = 0.0):
     """bfloat16 x [m, k] (or ``Prenormed``), interleaved gate/up weight [2i, k] -> bfloat16 [m, i] =
     silu(x g^T) * (x u^T), the gate applied to the float32 accumulators (no rounding in between).
-    With ``blocked_out`` the result comes as ``KBlocked`` when there are at most 16 rows and i % 32 == 0 (else as a tensor)."""
+    With ``blocked_out`` the result comes as ``KBlocked`` when there are at most 16 rows and i % 32 == 0 (else as a tensor).
+    ``slope``, ``limit``, ``up_offset``: the general gate of ``gated_act`` (g' * sigmoid(slope g') * (u' + up_offset)
+    with both branches limited when limit > 0) in the same epilogue; the defaults are SwiGLU."""
     if _backend is not None:
+        if (slope, limit, up_offset) != (1.0, 0.0, 0.0):
+            return _backend.linear_swiglu(x, w, blocked_out, slope, limit, up_offset)
         return _backend.linear_swiglu(x, w, blocked_out) if blocked_out else _backend.linear_swiglu(x, w)
     x, pre, mk, xl = _pre_args(x)
     wd, wl = _w_args(w)
@@ -561,7 +565,7 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
     scratch, nscratch = _splitk_scratch(x, m, n)
     _call("tp_linear_fused", _ptr(x), _ptr(wd), _BF16, _ptr(out.data if blocked_out else out), _BF16, 2, m, n, k, 1,
           _ptr(scratch), ctypes.c_size_t(nscratch), *pre, _ptr(None), _ptr(None), _ptr(None), (2 if blocked_out else 0) | wl | xl,
-          0, _ptr(None), _stream(), tag=(m, n, k))
+          0, _ptr(None), ctypes.c_float(slope), ctypes.c_float(limit), ctypes.c_float(up_offset), _stream(), tag=(m, n, k))
     return out
 
 
@@ -640,7 +644,8 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
          (partial_ok and residual is None and out_dtype == torch.float32))
     splits = ctypes.c_int(1)
     _call("tp_linear_fused", _ptr(x), _ptr(wd), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _ptr(scratch),
-          ctypes.c_size_t(nscratch), *pre, *post, layout, int(defer), ctypes.byref(splits), _stream(), tag=(m, n, k))
+          ctypes.c_size_t(nscratch), *pre, *post, layout, int(defer), ctypes.byref(splits), ctypes.c_float(1.0),
+          ctypes.c_float(0.0), ctypes.c_float(0.0), _stream(), tag=(m, n, k))
     if defer and splits.value > 1:
         if next_norm is None:
             return Partials(scratch[: splits.value * m * n].view(splits.value, m, n))

@@ -86,12 +86,21 @@ class GatedFFN(FeedForward):
     def load_weights(self, get):
         w = self.spec.weights
         gate, up = self._to_device(get(w["gate"])), self._to_device(get(w["up"]))
-        self.w13 = ops.tile_weight(torch.cat([gate, up], dim=0).contiguous())      # one product: gate columns, then up
+        # One product.  In bfloat16 the rows alternate eight of gate and eight of up, and the product's epilogue
+        # applies the activation to its float32 sums; else gate columns, then up columns, and a kernel of its own.
+        self.fused = self.dtype == torch.bfloat16 and ops.gated_layout_ok(self.intermediate_size, self.hidden_size)
+        if self.fused:
+            self.w13 = ops.tile_weight(ops.interleave_gate_up(gate, up))
+        else:
+            self.w13 = ops.tile_weight(torch.cat([gate, up], dim=0).contiguous())
         self.w2 = ops.tile_weight(self._to_device(get(w["down"])))
 
     def forward(self, x, ctx, residual=None):
-        gu = ops.linear(x, self.w13, torch.float32)
-        a = ops.gated_act(gu, self.dtype, self.slope, self.limit, self.up_offset)
+        if self.fused:
+            a = ops.linear_swiglu(x, self.w13, blocked_out=True, slope=self.slope, limit=self.limit, up_offset=self.up_offset)
+        else:
+            gu = ops.linear(x, self.w13, torch.float32)
+            a = ops.gated_act(gu, self.dtype, self.slope, self.limit, self.up_offset)
         return ops.linear(a, self.w2, torch.float32, residual=residual)
 
 

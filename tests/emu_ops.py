@@ -156,13 +156,15 @@ class EmuOps:
             return residual, Prenormed((residual * weight).to(torch.bfloat16), ss, eps)
         return y.to(out_dtype)
 
-    def linear_swiglu(self, x, w, blocked_out=False):
+    def linear_swiglu(self, x, w, blocked_out=False, slope=1.0, limit=0.0, up_offset=0.0):
         from tempura_amd.kernels.ops import KBlocked
         xd, scale = self._rows(x)
         x = xd
         y = ((x @ w.double().T) * scale).reshape(x.shape[0], -1, 2, 8)      # eight gate rows, eight up rows in turn
         g, u = y[:, :, 0].reshape(x.shape[0], -1), y[:, :, 1].reshape(x.shape[0], -1)
-        out = (g / (1.0 + torch.exp(-g)) * u).to(torch.bfloat16)
+        if limit > 0:
+            g, u = torch.clamp(g, max=limit), torch.clamp(u, -limit, limit)
+        out = (g / (1.0 + torch.exp(-slope * g)) * (u + up_offset)).to(torch.bfloat16)
         m, i = out.shape
         if blocked_out and 0 < m <= 16 and i % 32 == 0:
             return KBlocked(out.reshape(m, i // 8, 8).permute(1, 0, 2).contiguous(), m, i)

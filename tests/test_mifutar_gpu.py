@@ -413,3 +413,21 @@ def test_replay_program_on_a_model_folder(dirs, tmp_path):
     c = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(-1, vocab))
     assert not (out / "1.f32").exists()
     assert plain.logit_error(torch.cat([a, c]), torch.stack([ref[0], ref[10], ref[29], ref[3]])) < TOL["float32"]
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 40, 100, 300, 2048])
+def test_gated_product_with_limits_in_the_epilogue(m):
+    """The gate/up product that applies the limited activation to its float32 sums, at every number of rows that
+    takes another product kernel, against the product and the activation as two steps."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(m)
+    k, inter = 256, 384
+    x = (torch.randn(m, k, generator=g) * 1.5).to(torch.bfloat16)
+    gate, up = (torch.randn(inter, k, generator=g) * 0.1).to(torch.bfloat16), (torch.randn(inter, k, generator=g) * 0.1).to(torch.bfloat16)
+    w = ops.tile_weight(ops.interleave_gate_up(gate.to(DEV), up.to(DEV)))
+    for slope, limit, off in [(1.702, 1.5, 1.0), (1.0, 0.0, 0.0), (0.7, 0.4, -0.5)]:
+        got = ops.linear_swiglu(x.to(DEV), w, slope=slope, limit=limit, up_offset=off)
+        gu = torch.cat([x.double() @ gate.double().T, x.double() @ up.double().T], dim=1)
+        want = emu.gated_act(gu, torch.float64, slope, limit, off)
+        assert float(want.abs().max()) > 0.3
+        _close(got, want, 1e-2)
