@@ -381,6 +381,7 @@ extern "C" int tp_ssm_scan(const float* xbc, const float* proj, int proj_stride,
 // v = y * silu(z) (z: column z_col0 + j of the projection's rows), normed in `groups` equal parts, each by its own
 // root mean square (eps inside the root), times w [inner]; out [n, inner] float32 or bfloat16.
 // One block per (token, part).
+#define GN_ITEMS 8   // values a thread keeps between the sum and the store (parts up to 8 x the block)
 template <typename TO>
 __global__ void gated_group_norm_kernel(const float* __restrict__ y, const float* __restrict__ proj, int proj_stride,
                                         int z_col0, const float* __restrict__ w, float eps, TO* __restrict__ out, int inner,
@@ -389,6 +390,25 @@ __global__ void gated_group_norm_kernel(const float* __restrict__ y, const float
   const int t = blockIdx.x, q = blockIdx.y;
   const float* yr = y + (size_t)t * inner + (size_t)q * part;
   const float* zr = proj + (size_t)t * proj_stride + z_col0 + (size_t)q * part;
+  TO* o = out + (size_t)t * inner + (size_t)q * part;
+  const float* wr = w + (size_t)q * part;
+  if (part <= GN_ITEMS * (int)blockDim.x) {
+    float v[GN_ITEMS];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < GN_ITEMS; ++i) {
+      const int j = threadIdx.x + i * blockDim.x;
+      v[i] = j < part ? yr[j] * silu_f(zr[j]) : 0.f;
+      ss = fmaf(v[i], v[i], ss);
+    }
+    const float rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)part + eps);
+#pragma unroll
+    for (int i = 0; i < GN_ITEMS; ++i) {
+      const int j = threadIdx.x + i * blockDim.x;
+      if (j < part) from_float(o + j, v[i] * rstd * wr[j]);
+    }
+    return;
+  }
   float ss = 0.f;
   for (int j = threadIdx.x; j < part; j += blockDim.x) {
     const float v = yr[j] * silu_f(zr[j]);
@@ -396,8 +416,6 @@ __global__ void gated_group_norm_kernel(const float* __restrict__ y, const float
   }
   const float total = block_sum(ss, scratch);
   const float rstd = 1.0f / sqrtf(total / (float)part + eps);
-  TO* o = out + (size_t)t * inner + (size_t)q * part;
-  const float* wr = w + (size_t)q * part;
   for (int j = threadIdx.x; j < part; j += blockDim.x) from_float(o + j, yr[j] * silu_f(zr[j]) * rstd * wr[j]);
 }
 
