@@ -87,7 +87,7 @@ def test_stream_step(S, W, out_dtype):
 def test_gated_act_with_limits(out_dtype):
     ops = _ops()
     gu = torch.randn(7, 2 * 45, generator=torch.Generator().manual_seed(2)) * 3
-    for slope, limit, off in [(1.702, 1.5, 1.0), (1.0, 0.0, 0.0), (0.5, 0.25, -2.0)]:
+    for slope, limit, off in [(1.702, 1.25, 1.0), (1.0, 0.0, 0.0), (0.5, 0.25, -2.0)]:
         got = ops.gated_act(gu.to(DEV), out_dtype, slope, limit, off)
         _close(got, emu.gated_act(gu, out_dtype, slope, limit, off), 2e-6 if out_dtype == torch.float32 else 1e-2)
     logits = torch.randn(3, 11)
@@ -104,7 +104,7 @@ def _paged(n_ctx, kvh, d, ps, dtype, g):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,kvh,d,ps", [(4, 2, 16, 16), (3, 3, 10, 8), (8, 1, 96, 16), (2, 1, 64, 32)])
+@pytest.mark.parametrize("heads,kvh,d,ps", [(4, 2, 16, 16), (3, 3, 10, 8), (6, 2, 96, 16), (2, 1, 64, 32)])
 def test_biased_keys_as_values_into_the_cache(dtype, heads, kvh, d, ps):
     ops = _ops()
     g = torch.Generator().manual_seed(heads * 100 + d)
@@ -127,7 +127,7 @@ def test_biased_keys_as_values_into_the_cache(dtype, heads, kvh, d, ps):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,kvh,d,ps,window,L", [(4, 2, 16, 16, 7, 7), (3, 3, 10, 8, 20, 12), (8, 1, 96, 16, 136, 121),
+@pytest.mark.parametrize("heads,kvh,d,ps,window,L", [(4, 2, 16, 16, 7, 7), (3, 3, 10, 8, 20, 12), (6, 2, 96, 16, 100, 90),
                                                    (2, 1, 64, 16, 0, 30), (4, 4, 32, 16, 33, 33)])
 def test_attention_with_distance_bias_and_a_key_that_stands_out(dtype, heads, kvh, d, ps, window, L):
     """Portions behind a cached prefix and single tokens in one batch.  One key is made to dominate the scores of
@@ -207,7 +207,7 @@ def test_causal_conv_carries_its_inputs(channels, taps):
     assert torch.equal(s_dev.cpu()[3], state[3])            # a slot of no request is left alone
 
 
-@pytest.mark.parametrize("H,P,N,G", [(4, 8, 16, 2), (2, 24, 5, 1), (6, 48, 48, 2), (3, 64, 128, 3), (1, 40, 600, 1), (8, 16, 32, 1)])
+@pytest.mark.parametrize("H,P,N,G", [(4, 8, 16, 2), (2, 24, 5, 1), (6, 40, 56, 2), (3, 64, 128, 3), (1, 40, 600, 1), (8, 16, 32, 1)])
 def test_selective_scan_and_its_state(H, P, N, G):
     ops = _ops()
     g = torch.Generator().manual_seed(H * 10 + N)
@@ -264,7 +264,7 @@ def test_long_runs_in_pieces_side_by_side(H, P, N, G):
     assert torch.equal(s_dev.cpu()[5], state[5]) and torch.equal(s_dev.cpu()[:, :5], state[:, :5])
 
 
-@pytest.mark.parametrize("inner,groups", [(32, 1), (48, 3), (288, 2), (4096, 4)])
+@pytest.mark.parametrize("inner,groups", [(32, 1), (48, 3), (320, 2), (4096, 4)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 def test_gated_group_norm(inner, groups, out_dtype):
     ops = _ops()
@@ -425,7 +425,7 @@ def test_gated_product_with_limits_in_the_epilogue(m):
     x = (torch.randn(m, k, generator=g) * 1.5).to(torch.bfloat16)
     gate, up = (torch.randn(inter, k, generator=g) * 0.1).to(torch.bfloat16), (torch.randn(inter, k, generator=g) * 0.1).to(torch.bfloat16)
     w = ops.tile_weight(ops.interleave_gate_up(gate.to(DEV), up.to(DEV)))
-    for slope, limit, off in [(1.702, 1.5, 1.0), (1.0, 0.0, 0.0), (0.7, 0.4, -0.5)]:
+    for slope, limit, off in [(1.702, 1.25, 1.0), (1.0, 0.0, 0.0), (0.7, 0.4, -0.5)]:
         got = ops.linear_swiglu(x.to(DEV), w, slope=slope, limit=limit, up_offset=off)
         gu = torch.cat([x.double() @ gate.double().T, x.double() @ up.double().T], dim=1)
         want = emu.gated_act(gu, torch.float64, slope, limit, off)
