@@ -44,7 +44,7 @@ CASES: Dict[str, dict] = {
     # prompt here, no window at all, and a window of exactly one page
     "attn": {"architecture": "Mifutar", "vocab": 60, "width": 32, "streams": 1, "logit_scale": 2.0, "norm": {"eps": 1e-6},
              "layers": [_layer("attention", _attn(4, 1, 8, 500, 8, 64), 48, 1.0),
-                        _layer("attention", _attn(2, 2, 12, None, 4, 30), 40, 1.25),
+                        _layer("attention", _attn(2, 2, 12, None, 4, 30), 44, 1.25),      # (44: no multiple of eight)
                         _layer("attention", _attn(6, 3, 6, 16, 10, 16))]},
     # MFMA-friendly sizes: heads of 32 and 64, state 64, pages of 16 with windows at and beside page borders
     "wide": {"architecture": "Mifutar", "vocab": 96, "width": 128, "streams": 2, "logit_scale": 0.25, "norm": {"eps": 1e-5},
