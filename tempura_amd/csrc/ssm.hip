@@ -16,15 +16,17 @@ __device__ inline float silu_f(float v) { return v / (1.0f + expf(-v)); }
 __device__ inline float softplus_f(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 
 // ---- causal convolution per channel + SiLU ----------------------------------------------------
-// in: rows [n, in_stride] float32, the channels at column col0; w [channels, taps] (the last column is the current
-// token's), b [channels].  The inputs before a run's first token come from the request's state row (zeros for a
+// in: rows [n, in_stride] float32, the channels at column col0; w [taps, channels] (tap-major, so that the lanes of
+// a wave read neighbouring weights; the last tap is the current token's), b [channels].  The inputs before a run's first token come from the request's state row (zeros for a
 // fresh request).  out [n, channels] = silu(conv + b).
 __global__ void causal_conv_kernel(const float* __restrict__ in, int in_stride, int col0, const float* __restrict__ w,
                                    const float* __restrict__ b, const float* __restrict__ state, size_t state_stride,
                                    const int* __restrict__ cu_seqlens, const int* __restrict__ token_req,
-                                   const int* __restrict__ state_slots, float* __restrict__ out, int channels, int taps) {
-  const int t = blockIdx.x;
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+                                   const int* __restrict__ state_slots, float* __restrict__ out, int channels, int taps,
+                                   int channel_blocks) {
+  // (neighbouring blocks take neighbouring channels of one token: they read one row of the input after the other)
+  const int t = blockIdx.x / channel_blocks;
+  const int c = (blockIdx.x % channel_blocks) * blockDim.x + threadIdx.x;
   if (c >= channels) return;
   const int r = token_req[t];
   const int start = cu_seqlens[r];
@@ -34,7 +36,7 @@ __global__ void causal_conv_kernel(const float* __restrict__ in, int in_stride, 
   for (int k = 0; k < taps; ++k) {
     const int src = i - (taps - 1 - k);
     const float v = src >= 0 ? in[(size_t)(start + src) * in_stride + col0 + c] : st[(size_t)(taps - 1 + src) * channels + c];
-    acc = fmaf(w[(size_t)c * taps + k], v, acc);
+    acc = fmaf(w[(size_t)k * channels + c], v, acc);
   }
   out[(size_t)t * channels + c] = silu_f(acc);
 }
@@ -64,12 +66,12 @@ extern "C" int tp_causal_conv(const float* in, int in_stride, int col0, const fl
   TP_REQUIRE(in_stride >= col0 + channels && state_stride >= (size_t)(taps - 1) * channels, "causal_conv: rows too short");
   if (n == 0) return 0;
   const int threads = channels >= 256 ? 256 : 64;
-  const dim3 grid(n, (channels + threads - 1) / threads);
-  TP_REQUIRE(grid.y <= 65535, "causal_conv: too many channels");
-  hipLaunchKernelGGL(causal_conv_kernel, grid, dim3(threads), 0, s, in, in_stride, col0, w, b, state, state_stride,
-                     cu_seqlens, token_req, state_slots, out, channels, taps);
+  const int cb = (channels + threads - 1) / threads;
+  TP_REQUIRE(cb <= 65535 && (long)n * cb < 0x7fffffffL, "causal_conv: too many channels or tokens");
+  hipLaunchKernelGGL(causal_conv_kernel, dim3((unsigned)((long)n * cb)), dim3(threads), 0, s, in, in_stride, col0, w, b, state,
+                     state_stride, cu_seqlens, token_req, state_slots, out, channels, taps, cb);
   if (taps > 1 && n_req > 0)
-    hipLaunchKernelGGL(conv_state_kernel, dim3(n_req, grid.y), dim3(threads), 0, s, in, in_stride, col0, state,
+    hipLaunchKernelGGL(conv_state_kernel, dim3(n_req, cb), dim3(threads), 0, s, in, in_stride, col0, state,
                        state_stride, cu_seqlens, state_slots, channels, taps);
   TP_CHECK_LAUNCH("causal_conv");
   return 0;

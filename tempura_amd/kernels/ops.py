@@ -284,16 +284,16 @@ def qk_store(rows: torch.Tensor, q_bias: Optional[torch.Tensor], k_bias: Optiona
 def causal_conv(proj: torch.Tensor, col0: int, channels: int, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor,
                 cu_seqlens: torch.Tensor, token_req: torch.Tensor, state_slots: torch.Tensor, num_requests: int) -> torch.Tensor:
     """Causal convolution per channel over each request's run of tokens, then SiLU.  ``proj`` float32 [n, width]
-    holds the inputs at columns col0 .. col0 + channels; ``weight`` [channels, taps] (last column: the current
-    token), ``bias`` [channels]; ``state`` float32 [slots, row] whose rows start with the carried inputs
+    holds the inputs at columns col0 .. col0 + channels; ``weight`` [taps, channels] (tap-major; the last tap is the
+    current token's), ``bias`` [channels]; ``state`` float32 [slots, row] whose rows start with the carried inputs
     [taps - 1, channels] (oldest first) of the request in that slot: they are read for the first tokens of a run
     and replaced by the run's last inputs.  Returns float32 [n, channels]."""
     if _backend is not None:
         return _backend.causal_conv(proj, col0, channels, weight, bias, state, cu_seqlens, token_req, state_slots, num_requests)
     _dev_ok(proj, weight, bias, state, cu_seqlens, token_req, state_slots)
     _need(proj.dtype == torch.float32 and proj.dim() == 2 and 0 <= col0 and col0 + channels <= proj.shape[1], "causal_conv: bad rows")
-    _need(weight.dtype == torch.float32 and weight.dim() == 2 and weight.shape[0] == channels, "causal_conv: weight must be float32 [channels, taps]")
-    taps = weight.shape[1]
+    _need(weight.dtype == torch.float32 and weight.dim() == 2 and weight.shape[1] == channels, "causal_conv: weight must be float32 [taps, channels]")
+    taps = weight.shape[0]
     _need(bias.dtype == torch.float32 and bias.numel() == channels, "causal_conv: bias must be float32 [channels]")
     _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= (taps - 1) * channels, "causal_conv: state rows too short")
     n = proj.shape[0]

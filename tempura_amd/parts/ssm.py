@@ -73,7 +73,7 @@ class Mamba2Mixer(Mixer):
             w_in = torch.cat([w_in, torch.zeros((pad, w_in.shape[1]), dtype=w_in.dtype, device=w_in.device)], dim=0).contiguous()
         self.w_in = ops.tile_weight(w_in)
         f32 = lambda name: self._to_device(get(w[name]), torch.float32)
-        self.conv_w, self.conv_b = f32("conv"), f32("conv_bias")
+        self.conv_w, self.conv_b = f32("conv").t().contiguous(), f32("conv_bias")      # (tap-major for the kernel)
         self.dt_bias, self.a_log, self.d_skip = f32("dt_bias"), f32("a_log"), f32("d")
         self.norm_w = f32("norm")
         self.w_out = ops.tile_weight(self._to_device(get(w["out"])))

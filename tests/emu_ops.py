@@ -71,7 +71,7 @@ class EmuOps:
         return q.reshape(n, num_heads, head_dim).to(q_dtype).contiguous()
 
     def causal_conv(self, proj, col0, channels, weight, bias, state, cu_seqlens, token_req, state_slots, num_requests):
-        taps = weight.shape[1]
+        taps = weight.shape[0]                    # tap-major: [taps, channels]
         out = torch.zeros(proj.shape[0], channels, dtype=torch.float64)
         cu = cu_seqlens.tolist()
         for r in range(num_requests):
@@ -82,7 +82,7 @@ class EmuOps:
             carried = state[slot, : (taps - 1) * channels].double().reshape(taps - 1, channels)
             seq = torch.cat([carried, proj[a:b, col0: col0 + channels].double()], dim=0)
             for t in range(b - a):
-                out[a + t] = (seq[t: t + taps] * weight.double().T).sum(0) + bias.double()
+                out[a + t] = (seq[t: t + taps] * weight.double()).sum(0) + bias.double()
             state[slot, : (taps - 1) * channels] = seq[seq.shape[0] - (taps - 1):].reshape(-1).to(torch.float32)
         return (out * torch.sigmoid(out)).to(torch.float32)
 

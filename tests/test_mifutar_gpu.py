@@ -189,7 +189,7 @@ def test_causal_conv_carries_its_inputs(channels, taps):
     ops = _ops()
     g = torch.Generator().manual_seed(channels)
     col0, width = 11, 11 + channels + 6
-    w, b = torch.randn(channels, taps, generator=g), torch.randn(channels, generator=g)
+    w, b = torch.randn(taps, channels, generator=g), torch.randn(channels, generator=g)
     row = (taps - 1) * channels + 13
     state = torch.randn(5, row, generator=g)
     runs = [3, 1, 2, 9]                                     # shorter than, equal to and longer than taps - 1
@@ -353,6 +353,27 @@ def test_window_edge_decides_on_the_gpu(dirs, tmp_path, dtype):
     a = runner.step([StepEntry("r", toks[:60], list(range(60)))])
     rows = [a.clone()] + [runner.step([StepEntry("r", [t], [0])]).clone() for t in toks[60:]]
     assert plain.logit_error(torch.cat(rows).cpu(), ref) < tol
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompt_whole_and_in_portions(dirs, dtype):
+    """A prompt long enough that the recurrence runs in pieces side by side, whole and in portions that are cut
+    inside pieces, pages and windows, then decoded on; far keys and the state of hundreds of tokens decide here."""
+    from tempura_amd.engine.runner import StepEntry
+    toks = cases.tokens("wide", 560, 77)
+    ref = plain.forward(cases.config_json("wide"), cases.make_weights("wide"), toks)
+    want_rows = [0, 1, 255, 256, 257, 300, 511, 512, 540, 559]
+    for cuts in ([560], [300, 2, 129, 97, 31, 1]):
+        runner = _runner(dirs, "wide", dtype, 640)
+        runner.add_request("r")
+        rows, at = [], 0
+        for c in cuts:
+            w = [i - at for i in want_rows if at <= i < at + c]
+            lg = runner.step([StepEntry("r", toks[at: at + c], w)])
+            if w:
+                rows.append(lg.cpu().clone())
+            at += c
+        assert plain.logit_error(torch.cat(rows), ref[want_rows]) < TOL[dtype], cuts
 
 
 def test_long_decoding_through_a_captured_step(dirs):
