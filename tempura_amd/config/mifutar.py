@@ -65,7 +65,8 @@ class AttentionMixer:
         if mask is not None:
             if not isinstance(mask, dict):
                 raise ConfigError(f"config.json: {where}: 'mask' must be an object")
-            window = _num(mask, "size", where + ".mask")
+            if mask.get("size") is not None:
+                window = _num(mask, "size", where + ".mask")
         m = cls(_num(d, "heads", where), _num(d, "kv_heads", where), _num(d, "dim", where),
                 _num(d, "vdim", where) if d.get("vdim") is not None else _num(d, "dim", where),
                 _num(d, "scale", where, float), _num(d, "bias_max", where), window,
