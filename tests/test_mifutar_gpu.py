@@ -128,7 +128,8 @@ def test_biased_keys_as_values_into_the_cache(dtype, heads, kvh, d, ps):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kvh,d,ps,window,L", [(4, 2, 16, 16, 7, 7), (3, 3, 10, 8, 20, 12), (6, 2, 96, 16, 100, 90),
-                                                   (2, 1, 64, 16, 0, 30), (4, 4, 32, 16, 33, 33)])
+                                                   (2, 1, 64, 16, 0, 30), (4, 4, 32, 16, 33, 33), (8, 2, 128, 16, 100, 64),
+                                                   (2, 1, 64, 16, 0, 1500), (5, 1, 128, 32, 120, 121)])
 def test_attention_with_distance_bias_and_a_key_that_stands_out(dtype, heads, kvh, d, ps, window, L):
     """Portions behind a cached prefix and single tokens in one batch.  One key is made to dominate the scores of
     the queries that may see it: at the window's last place for one request, one place outside it for another, and
