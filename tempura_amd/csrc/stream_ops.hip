@@ -168,17 +168,21 @@ extern "C" int tp_scale_f32(float* x, size_t n, float scale, hipStream_t s) {
 }
 
 // ---- gated activation with limits -------------------------------------------------------------
-// gu [m, 2 I] (gate columns, then up columns): g = min(gate, limit), u = clamp(up, -limit, limit) (limit <= 0: no
-// limits), out = g * sigmoid(slope * g) * (u + up_offset).  slope 1, no limit and offset 0 is SwiGLU.
+// gu [m, 2 I] (gate columns, then up columns; or, interleaved, eight gate columns and eight up columns in turn, as
+// the products with the activation in their epilogue have their weights): g = min(gate, limit),
+// u = clamp(up, -limit, limit) (limit <= 0: no limits), out = g * sigmoid(slope * g) * (u + up_offset).
+// slope 1, no limit and offset 0 is SwiGLU.
 template <typename TI, typename TO>
 __global__ void gated_act_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter, size_t total, float slope,
-                                 float limit, float up_offset) {
+                                 float limit, float up_offset, int interleaved) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t m = idx / inter;
   const int i = (int)(idx % inter);
-  float g = to_float(gu[m * 2 * inter + i]);
-  float u = to_float(gu[m * 2 * inter + inter + i]);
+  const int gc = interleaved ? (i / 8) * 16 + i % 8 : i;
+  const int uc = interleaved ? gc + 8 : inter + i;
+  float g = to_float(gu[m * 2 * inter + gc]);
+  float u = to_float(gu[m * 2 * inter + uc]);
   if (limit > 0.f) {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
@@ -187,14 +191,14 @@ __global__ void gated_act_kernel(const TI* __restrict__ gu, TO* __restrict__ out
 }
 
 extern "C" int tp_gated_act(const void* gu, int in_dt, void* out, int out_dt, int m, int inter, float slope, float limit,
-                            float up_offset, hipStream_t s) {
-  TP_REQUIRE(m >= 0 && inter > 0, "gated_act: bad sizes");
+                            float up_offset, int interleaved, hipStream_t s) {
+  TP_REQUIRE(m >= 0 && inter > 0 && (!interleaved || inter % 8 == 0), "gated_act: bad sizes");
   if (m == 0) return 0;
   const size_t total = (size_t)m * inter;
   const dim3 grid((unsigned)((total + 255) / 256));
 #define LAUNCH(TI, TO)                                                                                         \
   hipLaunchKernelGGL((gated_act_kernel<TI, TO>), grid, dim3(256), 0, s, (const TI*)gu, (TO*)out, inter, total, slope, \
-                     limit, up_offset)
+                     limit, up_offset, interleaved)
   if (in_dt == TP_F32 && out_dt == TP_F32)
     LAUNCH(float, float);
   else if (in_dt == TP_F32 && out_dt == TP_BF16)

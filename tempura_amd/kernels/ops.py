@@ -234,17 +234,19 @@ def scale_(x: torch.Tensor, scale: float) -> torch.Tensor:
     return x
 
 
-def gated_act(gu: torch.Tensor, out_dtype: torch.dtype, slope: float = 1.0, limit: float = 0.0, up_offset: float = 0.0) -> torch.Tensor:
-    """[m, 2i] (gate columns then up columns) -> out_dtype [m, i]: g = min(gate, limit), u = clamp(up, -limit, limit)
+def gated_act(gu: torch.Tensor, out_dtype: torch.dtype, slope: float = 1.0, limit: float = 0.0, up_offset: float = 0.0,
+              interleaved: bool = False) -> torch.Tensor:
+    """[m, 2i] (gate columns then up columns; ``interleaved``: eight gate and eight up columns in turn, the layout of
+    ``interleave_gate_up``) -> out_dtype [m, i]: g = min(gate, limit), u = clamp(up, -limit, limit)
     (limit <= 0: none), g * sigmoid(slope * g) * (u + up_offset)."""
     if _backend is not None:
-        return _backend.gated_act(gu, out_dtype, slope, limit, up_offset)
+        return _backend.gated_act(gu, out_dtype, slope, limit, up_offset, interleaved)
     _dev_ok(gu)
     _need(gu.dim() == 2 and gu.shape[1] % 2 == 0, "gated_act: input must be [m, 2i]")
     m, i2 = gu.shape
     out = torch.empty((m, i2 // 2), dtype=out_dtype, device=gu.device)
     _call("tp_gated_act", _ptr(gu), _dt(gu), _ptr(out), _dtcode(out_dtype), m, i2 // 2, ctypes.c_float(slope),
-          ctypes.c_float(limit), ctypes.c_float(up_offset), _stream())
+          ctypes.c_float(limit), ctypes.c_float(up_offset), int(bool(interleaved)), _stream())
     return out
 
 
@@ -383,6 +385,11 @@ def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
 
 #: bfloat16 products may use the matrix-core kernels (tests switch this off to grade the general kernel)
 allow_mfma = True
+
+
+#: a gate with constants of its own runs in the product's epilogue from this many rows on (the products of fewer
+#: rows stream the weights once and have the plain gated SiLU only)
+gated_epilogue_rows = 17
 
 
 def gated_layout_ok(n_rows: int, k: int) -> bool:
@@ -543,7 +550,8 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False, slope: float = 
     silu(x g^T) * (x u^T), the gate applied to the float32 accumulators (no rounding in between).
     With ``blocked_out`` the result comes as ``KBlocked`` when there are at most 16 rows and i % 32 == 0 (else as a tensor).
     ``slope``, ``limit``, ``up_offset``: the general gate of ``gated_act`` (g' * sigmoid(slope g') * (u' + up_offset)
-    with both branches limited when limit > 0) in the same epilogue; the defaults are SwiGLU."""
+    with both branches limited when limit > 0) in the same epilogue; the defaults are SwiGLU.  The products of at
+    most 16 rows have the default gate only (``gated_epilogue_rows``)."""
     if _backend is not None:
         if (slope, limit, up_offset) != (1.0, 0.0, 0.0):
             return _backend.linear_swiglu(x, w, blocked_out, slope, limit, up_offset)

@@ -96,11 +96,12 @@ class GatedFFN(FeedForward):
         self.w2 = ops.tile_weight(self._to_device(get(w["down"])))
 
     def forward(self, x, ctx, residual=None):
-        if self.fused:
-            a = ops.linear_swiglu(x, self.w13, blocked_out=True, slope=self.slope, limit=self.limit, up_offset=self.up_offset)
+        if self.fused and x.shape[0] >= ops.gated_epilogue_rows:
+            a = ops.linear_swiglu(x, self.w13, slope=self.slope, limit=self.limit, up_offset=self.up_offset)
         else:
+            # (a few rows, or sizes the fused product does not take: the product's float32 sums, then the activation)
             gu = ops.linear(x, self.w13, torch.float32)
-            a = ops.gated_act(gu, self.dtype, self.slope, self.limit, self.up_offset)
+            a = ops.gated_act(gu, self.dtype, self.slope, self.limit, self.up_offset, interleaved=self.fused)
         return ops.linear(a, self.w2, torch.float32, residual=residual)
 
 

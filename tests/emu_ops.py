@@ -44,9 +44,13 @@ class EmuOps:
         x.mul_(scale)
         return x
 
-    def gated_act(self, gu, out_dtype, slope=1.0, limit=0.0, up_offset=0.0):
+    def gated_act(self, gu, out_dtype, slope=1.0, limit=0.0, up_offset=0.0, interleaved=False):
         i = gu.shape[1] // 2
-        g, u = gu.double()[:, :i], gu.double()[:, i:]
+        if interleaved:
+            y = gu.double().reshape(gu.shape[0], -1, 2, 8)
+            g, u = y[:, :, 0].reshape(gu.shape[0], -1), y[:, :, 1].reshape(gu.shape[0], -1)
+        else:
+            g, u = gu.double()[:, :i], gu.double()[:, i:]
         if limit > 0:
             g = torch.clamp(g, max=limit)
             u = torch.clamp(u, -limit, limit)
