@@ -11,9 +11,9 @@ The names a user starts from (the reference's ``InferenceModel`` and ``inspect``
 """
 __version__ = "0.1.0"
 
-from .config import PRESETS, LlamaConfig, MifutarConfig, load_config          # noqa: E402,F401
+from .config import PRESETS, BomotarConfig, LlamaConfig, MifutarConfig, load_config          # noqa: E402,F401
 from .sampling import SamplingParams                           # noqa: E402,F401
 from .engine import Engine                                     # noqa: E402,F401
 from .inspect import inspect                                   # noqa: E402,F401  (the function, which now hides the module of its name)
 
-__all__ = ["Engine", "SamplingParams", "LlamaConfig", "MifutarConfig", "PRESETS", "load_config", "inspect", "__version__"]
+__all__ = ["Engine", "SamplingParams", "LlamaConfig", "MifutarConfig", "BomotarConfig", "PRESETS", "load_config", "inspect", "__version__"]

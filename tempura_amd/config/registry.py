@@ -13,6 +13,7 @@ from typing import Any, Callable, Dict
 
 from .llama import ConfigError, LlamaConfig
 from .mifutar import MifutarConfig
+from .bomotar import BomotarConfig
 
 _ARCHITECTURES: Dict[str, Any] = {}
 
@@ -72,3 +73,4 @@ def config_from_file(path: str):
 register_architecture("LlamaForCausalLM", LlamaConfig)
 register_architecture("llama", LlamaConfig)
 register_architecture("Mifutar", MifutarConfig)
+register_architecture("Bomotar", BomotarConfig)

@@ -24,7 +24,8 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_seqlens,
     const int* __restrict__ context_lens, const int* __restrict__ token_req, T* __restrict__ out, int n_heads,
-    int n_kv, int head_dim, int page_size, float scale, int window, const float* __restrict__ dist_bias, int bias_len) {
+    int n_kv, int head_dim, int page_size, float scale, int window, const float* __restrict__ dist_bias, int bias_len,
+    int value_dim) {
   extern __shared__ float qs[];  // the query row, float32
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = token_req[t];
@@ -70,20 +71,20 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
     for (int jj = 0; jj < n_valid; ++jj) {
       const float pj = __shfl(p, jj, TP_WAVE);
       const int vb = __shfl(vbase, jj, TP_WAVE);
-      const T* vr = v_cache + (size_t)vb * head_dim * page_size + (j0 + jj) % page_size;
+      const T* vr = v_cache + (size_t)vb * value_dim * page_size + (j0 + jj) % page_size;
 #pragma unroll
       for (int i = 0; i < ATT_MAX_ACC; ++i) {
         const int d = lane + i * TP_WAVE;
-        if (d < head_dim) acc[i] = fmaf(pj, to_float(vr[(size_t)d * page_size]), acc[i]);
+        if (d < value_dim) acc[i] = fmaf(pj, to_float(vr[(size_t)d * page_size]), acc[i]);
       }
     }
   }
   const float inv = 1.0f / l;
-  T* o = out + ((size_t)t * n_heads + h) * head_dim;
+  T* o = out + ((size_t)t * n_heads + h) * value_dim;
 #pragma unroll
   for (int i = 0; i < ATT_MAX_ACC; ++i) {
     const int d = lane + i * TP_WAVE;
-    if (d < head_dim) from_float(o + d, acc[i] * inv);
+    if (d < value_dim) from_float(o + d, acc[i] * inv);
   }
 }
 
@@ -101,7 +102,11 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
                                   int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale,
                                   int window, int max_q_len, int max_ctx, int allow_fast, int num_single,
                                   int num_splits, float* scratch, int portion_splits, int portion_min_steps,
-                                  float* portion_scratch, const float* dist_bias, int bias_len, hipStream_t s) {
+                                  float* portion_scratch, const float* dist_bias, int bias_len, int value_dim,
+                                  hipStream_t s) {
+  // value_dim: the size of a value head (0: head_dim): v_cache is [page, kv_head, value_dim, page_size] and out
+  // [n, heads * value_dim]; the matrix-core kernels take equal sizes only.
+  if (value_dim <= 0) value_dim = head_dim;
   // num_single: how many requests bring exactly one token (they go to the split decode kernel,
   // which, with more than one split, needs `scratch` of n_req * n_heads * num_splits * (head_dim + 2)
   // floats).  portion_splits > 1: the keys of every longer request are split over that many blocks,
@@ -109,13 +114,13 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
   TP_REQUIRE(n_tokens >= 0 && n_req >= 0 && n_heads > 0 && n_kv > 0 && head_dim > 0 && page_size > 0,
              "paged_attention: bad sizes");
   TP_REQUIRE(n_heads % n_kv == 0, "paged_attention: %d heads is not a multiple of %d kv heads", n_heads, n_kv);
-  TP_REQUIRE(head_dim <= TP_WAVE * ATT_MAX_ACC, "paged_attention: head_dim %d exceeds %d", head_dim,
-             TP_WAVE * ATT_MAX_ACC);
+  TP_REQUIRE(head_dim <= TP_WAVE * ATT_MAX_ACC && value_dim <= TP_WAVE * ATT_MAX_ACC, "paged_attention: head size %d / %d exceeds %d",
+             head_dim, value_dim, TP_WAVE * ATT_MAX_ACC);
   TP_REQUIRE(window >= 0, "paged_attention: window must be >= 0");
   TP_REQUIRE(n_heads <= 65535, "paged_attention: too many heads");
   if (n_tokens == 0) return 0;
   TP_REQUIRE(dist_bias == nullptr || bias_len > 0, "paged_attention: empty distance bias table");
-  if (dt == TP_BF16 && allow_fast) {
+  if (dt == TP_BF16 && allow_fast && value_dim == head_dim) {
     const int rc = tp_paged_attention_fast(q, k_cache, v_cache, block_tables, table_width, cu_seqlens,
                                            context_lens, out, n_tokens, n_req, n_heads, n_kv, head_dim,
                                            page_size, scale, window, max_q_len, num_single, num_splits, scratch, token_req,
@@ -127,11 +132,11 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
   if (dt == TP_F32)
     hipLaunchKernelGGL(paged_attention_kernel<float>, grid, dim3(64), shmem, s, (const float*)q,
                        (const float*)k_cache, (const float*)v_cache, block_tables, table_width, cu_seqlens,
-                       context_lens, token_req, (float*)out, n_heads, n_kv, head_dim, page_size, scale, window, dist_bias, bias_len);
+                       context_lens, token_req, (float*)out, n_heads, n_kv, head_dim, page_size, scale, window, dist_bias, bias_len, value_dim);
   else if (dt == TP_BF16)
     hipLaunchKernelGGL(paged_attention_kernel<bf16_t>, grid, dim3(64), shmem, s, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_seqlens,
-                       context_lens, token_req, (bf16_t*)out, n_heads, n_kv, head_dim, page_size, scale, window, dist_bias, bias_len);
+                       context_lens, token_req, (bf16_t*)out, n_heads, n_kv, head_dim, page_size, scale, window, dist_bias, bias_len, value_dim);
   else
     TP_REQUIRE(false, "paged_attention: unknown dtype %d", dt);
   TP_CHECK_LAUNCH("paged_attention");

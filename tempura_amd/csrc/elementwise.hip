@@ -353,8 +353,12 @@ __global__ void value_write_kernel(const float* __restrict__ qkv, int row_stride
 extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* positions, const int* slots,
                                 const double* inv_freq, int rotary_dim, float factor, int n, int n_heads,
                                 int n_kv, int head_dim, void* q_out, int q_dt, void* k_cache, void* v_cache,
-                                int cache_dt, int page_size, int splits, const float* cos_sin, hipStream_t s) {
+                                int cache_dt, int page_size, int splits, const float* cos_sin, int value_dim,
+                                hipStream_t s) {
+  // value_dim: the size of a value head (0: head_dim); the value cache is [page, kv_head, value_dim, page_size]
+  if (value_dim <= 0) value_dim = head_dim;
   TP_REQUIRE(n >= 0 && n_heads > 0 && n_kv >= 0 && head_dim > 0, "rope_kv_write: bad sizes");
+  TP_REQUIRE(value_dim <= 1024, "rope_kv_write: value size %d exceeds 1024", value_dim);
   TP_REQUIRE(splits >= 1 && splits <= 16, "rope_kv_write: bad number of partial sums");
   const size_t split_stride = (size_t)n * row_stride;   // qkv is [splits, n, row_stride]
   TP_REQUIRE(head_dim % 2 == 0 && head_dim <= 1024, "rope_kv_write: head_dim %d must be even and <= 1024", head_dim);
@@ -362,14 +366,16 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
              "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rotary_dim, head_dim);
   TP_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "rope_kv_write: no frequency table");
   TP_REQUIRE(slots == nullptr || (k_cache && v_cache && page_size > 0), "rope_kv_write: cache missing");
-  TP_REQUIRE(row_stride >= (n_heads + (slots ? 2 * n_kv : 0)) * head_dim, "rope_kv_write: row too short");
+  TP_REQUIRE(row_stride >= (n_heads + (slots ? n_kv : 0)) * head_dim + (slots ? n_kv * value_dim : 0), "rope_kv_write: row too short");
   if (n == 0) return 0;
   const int pairs = head_dim / 2;
   const int threads = pairs <= 256 ? 256 : 512;
   const int hpb = threads / pairs;
   // long steps (prompt portions, mostly) write their values sixteen tokens at a time (value_write_kernel);
   // a batch of single decoded tokens has no runs, and a second kernel would only cost it a launch
-  const bool grouped_values = slots != nullptr && n >= 256 && n_kv <= 65535;
+  // (values of another size than the keys always go through it: the rotation kernel walks heads of head_dim)
+  const bool grouped_values = slots != nullptr && (n >= 256 || value_dim != head_dim) && n_kv <= 65535;
+  TP_REQUIRE(slots == nullptr || value_dim == head_dim || grouped_values, "rope_kv_write: too many key heads");
   const int total_heads = n_heads + (slots ? (grouped_values ? 1 : 2) * n_kv : 0);
   const dim3 grid(n, (total_heads + hpb - 1) / hpb);
   TP_REQUIRE(grid.y <= 65535, "rope_kv_write: too many heads");
@@ -416,11 +422,11 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
     const dim3 vgrid((n + 15) / 16, n_kv);
     const int v_col0 = (n_heads + n_kv) * head_dim;
     if (cache_dt == TP_BF16)
-      hipLaunchKernelGGL((value_write_kernel<bf16_t>), vgrid, dim3((head_dim + 63) / 64 * 64), 0, s, qkv, row_stride, slots, n,
-                         v_col0, n_kv, head_dim, (bf16_t*)v_cache, page_size, splits, split_stride);
+      hipLaunchKernelGGL((value_write_kernel<bf16_t>), vgrid, dim3((value_dim + 63) / 64 * 64), 0, s, qkv, row_stride, slots, n,
+                         v_col0, n_kv, value_dim, (bf16_t*)v_cache, page_size, splits, split_stride);
     else
-      hipLaunchKernelGGL((value_write_kernel<float>), vgrid, dim3((head_dim + 63) / 64 * 64), 0, s, qkv, row_stride, slots, n,
-                         v_col0, n_kv, head_dim, (float*)v_cache, page_size, splits, split_stride);
+      hipLaunchKernelGGL((value_write_kernel<float>), vgrid, dim3((value_dim + 63) / 64 * 64), 0, s, qkv, row_stride, slots, n,
+                         v_col0, n_kv, value_dim, (float*)v_cache, page_size, splits, split_stride);
   }
   TP_CHECK_LAUNCH("rope_kv_write");
   return 0;

@@ -1,0 +1,326 @@
+// Small kernels around the products of a layer: an embedding with a hashed bigram table, the gate on an attention's
+// output, the norm behind a sublayer added into the residual stream, a plain activation, and the router of a
+// mixture of experts with the weighted sum of its experts' outputs.  Float32 arithmetic throughout; a row's result
+// never depends on other rows.
+#include <math.h>
+
+#include "common.h"
+
+__device__ inline float l_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
+
+// ---- embedding plus a row of a hashed bigram table --------------------------------------------
+// out[t] = table[token] + bigram[row], row = (previous * mul_prev + token * mul_cur) mod buckets, and row `buckets`
+// (the table's last) for the token at position 0.  The previous token is the one before it in the step's run, or,
+// for a run's first token, what the request's state row holds; a second kernel leaves each run's last token there.
+template <typename T>
+__global__ void embed_bigram_kernel(const int* __restrict__ tokens, const int* __restrict__ positions,
+                                    const int* __restrict__ token_req, const int* __restrict__ cu_seqlens,
+                                    const int* __restrict__ state_slots, const int* __restrict__ prev_state,
+                                    const T* __restrict__ table, const T* __restrict__ bigram, float* __restrict__ out,
+                                    int hidden, long long mul_prev, long long mul_cur, long long buckets) {
+  const int t = blockIdx.x;
+  const int tok = tokens[t];
+  long long row = buckets;
+  if (positions[t] != 0) {
+    const int r = token_req[t];
+    const int prev = t > cu_seqlens[r] ? tokens[t - 1] : prev_state[state_slots[r]];
+    row = ((long long)prev * mul_prev + (long long)tok * mul_cur) % buckets;
+  }
+  const T* a = table + (size_t)tok * hidden;
+  const T* b = bigram + (size_t)row * hidden;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) out[(size_t)t * hidden + c] = to_float(a[c]) + to_float(b[c]);
+}
+
+__global__ void last_token_kernel(const int* __restrict__ tokens, const int* __restrict__ cu_seqlens,
+                                  const int* __restrict__ state_slots, int* __restrict__ prev_state, int n_req) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n_req) return;
+  const int end = cu_seqlens[r + 1];
+  if (end > cu_seqlens[r]) prev_state[state_slots[r]] = tokens[end - 1];
+}
+
+extern "C" int tp_embed_bigram(const int* tokens, const int* positions, const int* token_req, const int* cu_seqlens,
+                               const int* state_slots, int* prev_state, const void* table, const void* bigram, int dt,
+                               float* out, int n, int n_req, int hidden, long long mul_prev, long long mul_cur,
+                               long long buckets, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && n_req >= 0 && hidden > 0 && buckets > 0 && mul_prev >= 0 && mul_cur >= 0, "embed_bigram: bad sizes");
+  if (n == 0) return 0;
+  const int threads = hidden >= 256 ? 256 : 64;
+  if (dt == TP_F32)
+    hipLaunchKernelGGL(embed_bigram_kernel<float>, dim3(n), dim3(threads), 0, s, tokens, positions, token_req, cu_seqlens,
+                       state_slots, prev_state, (const float*)table, (const float*)bigram, out, hidden, mul_prev, mul_cur, buckets);
+  else if (dt == TP_BF16)
+    hipLaunchKernelGGL(embed_bigram_kernel<bf16_t>, dim3(n), dim3(threads), 0, s, tokens, positions, token_req, cu_seqlens,
+                       state_slots, prev_state, (const bf16_t*)table, (const bf16_t*)bigram, out, hidden, mul_prev, mul_cur, buckets);
+  else
+    TP_REQUIRE(false, "embed_bigram: unknown dtype %d", dt);
+  if (n_req > 0)
+    hipLaunchKernelGGL(last_token_kernel, dim3((n_req + 63) / 64), dim3(64), 0, s, tokens, cu_seqlens, state_slots, prev_state, n_req);
+  TP_CHECK_LAUNCH("embed_bigram");
+  return 0;
+}
+
+// ---- gate on a mixer's output -----------------------------------------------------------------
+// out[t, out_col0 + c] = a[t, c] * sigmoid(proj[t, gate_col0 + c]) * scale (no gate: a * scale); the product is
+// formed in float32 and rounded once.
+template <typename T>
+__global__ void sigmoid_gate_kernel(const T* __restrict__ a, const float* __restrict__ proj, int proj_stride, int gate_col0,
+                                    float scale, T* __restrict__ out, int out_stride, int out_col0, int width, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / width;
+  const int c = (int)(i % width);
+  float v = to_float(a[i]);
+  if (proj != nullptr) v *= l_sigmoid(proj[t * proj_stride + gate_col0 + c]);
+  from_float(out + t * out_stride + out_col0 + c, v * scale);
+}
+
+extern "C" int tp_sigmoid_gate(const void* a, int dt, const float* proj, int proj_stride, int gate_col0, float scale, void* out,
+                               int out_stride, int out_col0, int n, int width, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && width > 0 && out_col0 >= 0 && out_stride >= out_col0 + width, "sigmoid_gate: bad sizes");
+  TP_REQUIRE(proj == nullptr || (gate_col0 >= 0 && proj_stride >= gate_col0 + width), "sigmoid_gate: gate rows too short");
+  if (n == 0) return 0;
+  const size_t total = (size_t)n * width;
+  const dim3 grid((unsigned)((total + 255) / 256));
+  if (dt == TP_F32)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, grid, dim3(256), 0, s, (const float*)a, proj, proj_stride, gate_col0, scale,
+                       (float*)out, out_stride, out_col0, width, total);
+  else if (dt == TP_BF16)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)a, proj, proj_stride, gate_col0, scale,
+                       (bf16_t*)out, out_stride, out_col0, width, total);
+  else
+    TP_REQUIRE(false, "sigmoid_gate: unknown dtype %d", dt);
+  TP_CHECK_LAUNCH("sigmoid_gate");
+  return 0;
+}
+
+// ---- a sublayer's output, normed, into the residual stream ------------------------------------
+// h[t] += y[t] / sqrt(mean(y[t]^2) + eps) * w; then, with w_next, the next sublayer's input
+// x[t] = h[t] / sqrt(mean(h[t]^2) + eps_next) * w_next as TO.  One block per row.
+template <typename TO>
+__global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ h, const float* __restrict__ y,
+                                                       const float* __restrict__ w, float eps,
+                                                       const float* __restrict__ w_next, float eps_next,
+                                                       TO* __restrict__ x, int width) {
+  __shared__ float scratch[32];
+  const size_t base = (size_t)blockIdx.x * width;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) ss = fmaf(y[base + c], y[base + c], ss);
+  ss = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(ss / (float)width + eps);
+  float ss2 = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = h[base + c] + y[base + c] * rstd * w[c];
+    h[base + c] = v;
+    ss2 = fmaf(v, v, ss2);
+  }
+  if (w_next == nullptr) return;
+  ss2 = block_sum(ss2, scratch);
+  const float rstd2 = 1.0f / sqrtf(ss2 / (float)width + eps_next);
+  // (each thread reads back what it wrote itself)
+  for (int c = threadIdx.x; c < width; c += blockDim.x) from_float(x + base + c, h[base + c] * rstd2 * w_next[c]);
+}
+
+extern "C" int tp_norm_add(float* h, const float* y, const float* w, float eps, const float* w_next, float eps_next, void* x,
+                           int x_dt, int n, int width, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && width > 0, "norm_add: bad sizes");
+  TP_REQUIRE(w_next == nullptr || x != nullptr, "norm_add: no place for the next rows");
+  if (n == 0) return 0;
+  const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+  if (w_next == nullptr || x_dt == TP_F32)
+    hipLaunchKernelGGL(norm_add_kernel<float>, dim3(n), dim3(threads), 0, s, h, y, w, eps, w_next, eps_next, (float*)x, width);
+  else if (x_dt == TP_BF16)
+    hipLaunchKernelGGL(norm_add_kernel<bf16_t>, dim3(n), dim3(threads), 0, s, h, y, w, eps, w_next, eps_next, (bf16_t*)x, width);
+  else
+    TP_REQUIRE(false, "norm_add: unknown dtype %d", x_dt);
+  TP_CHECK_LAUNCH("norm_add");
+  return 0;
+}
+
+// ---- a plain activation -----------------------------------------------------------------------
+// kind 0: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))); kind 1: SiLU.
+template <typename TI, typename TO>
+__global__ void activation_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t total, int kind) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const float z = to_float(in[i]);
+  float v;
+  if (kind == 0)
+    v = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  else
+    v = z * l_sigmoid(z);
+  from_float(out + i, v);
+}
+
+extern "C" int tp_activation(const void* in, int in_dt, void* out, int out_dt, size_t total, int kind, hipStream_t s) {
+  TP_REQUIRE(kind == 0 || kind == 1, "activation: unknown kind %d", kind);
+  if (total == 0) return 0;
+  const dim3 grid((unsigned)((total + 255) / 256));
+#define ACT(TI, TO) hipLaunchKernelGGL((activation_kernel<TI, TO>), grid, dim3(256), 0, s, (const TI*)in, (TO*)out, total, kind)
+  if (in_dt == TP_F32 && out_dt == TP_F32)
+    ACT(float, float);
+  else if (in_dt == TP_F32 && out_dt == TP_BF16)
+    ACT(float, bf16_t);
+  else if (in_dt == TP_BF16 && out_dt == TP_BF16)
+    ACT(bf16_t, bf16_t);
+  else
+    TP_REQUIRE(false, "activation: unsupported dtypes %d -> %d", in_dt, out_dt);
+#undef ACT
+  TP_CHECK_LAUNCH("activation");
+  return 0;
+}
+
+// ---- router of a mixture of experts -----------------------------------------------------------
+// logits [n, logit_stride] float32 (the first `experts` columns count).  s = softmax over the experts; the choice
+// score of expert e is s[e] + correction[e]; experts form `groups` equal groups of neighbours, a group's score is
+// its largest choice score, and only experts of the `keep` best groups can be chosen (groups <= 1: all); the `top`
+// allowed experts with the largest choice scores are chosen (ties: the lower index), and a chosen expert's weight
+// is s[e].  dense [n, experts] gets the weight of every chosen expert and 0 elsewhere; ids and weights [n, top]
+// list the chosen experts in the order of choice.  One wave per token; lane l holds experts l, l + 64, ...
+#define ROUTE_PER_LANE 8   // experts <= 64 * ROUTE_PER_LANE
+
+__device__ inline void wave_arg_best(float& v, int& i) {
+#pragma unroll
+  for (int o = TP_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, TP_WAVE);
+    const int oi = __shfl_xor(i, o, TP_WAVE);
+    if (ov > v || (ov == v && oi < i)) {
+      v = ov;
+      i = oi;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int logit_stride,
+                                                        const float* __restrict__ correction, int experts, int top,
+                                                        int groups, int keep, float* __restrict__ dense,
+                                                        int* __restrict__ ids, float* __restrict__ weights, int n) {
+  extern __shared__ float lds[];   // per wave: choice scores [experts], then group scores [groups]
+  const int wave = threadIdx.x / TP_WAVE, lane = threadIdx.x % TP_WAVE;
+  // (a wave past the last token works on the last token again and stores nothing: every wave reaches every barrier)
+  const bool live = blockIdx.x * 4 + wave < n;
+  const int t = live ? blockIdx.x * 4 + wave : n - 1;
+  float* choice_l = lds + (size_t)wave * (experts + max(groups, 1));
+  float* group_l = choice_l + experts;
+  float z[ROUTE_PER_LANE], sc[ROUTE_PER_LANE], ch[ROUTE_PER_LANE];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int k = 0; k < ROUTE_PER_LANE; ++k) {
+    const int e = lane + k * TP_WAVE;
+    z[k] = e < experts ? logits[(size_t)t * logit_stride + e] : -INFINITY;
+    mx = fmaxf(mx, z[k]);
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < ROUTE_PER_LANE; ++k) {
+    sc[k] = lane + k * TP_WAVE < experts ? expf(z[k] - mx) : 0.f;
+    sum += sc[k];
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int k = 0; k < ROUTE_PER_LANE; ++k) {
+    const int e = lane + k * TP_WAVE;
+    sc[k] *= inv;
+    ch[k] = e < experts ? sc[k] + correction[e] : -INFINITY;
+    if (e < experts) {
+      choice_l[e] = ch[k];
+      if (live) dense[(size_t)t * experts + e] = 0.f;
+    }
+  }
+  if (groups > 1) {
+    const int per = experts / groups;
+    __syncthreads();
+    for (int g = lane; g < groups; g += TP_WAVE) {
+      float best = -INFINITY;
+      for (int i = 0; i < per; ++i) best = fmaxf(best, choice_l[g * per + i]);
+      group_l[g] = best;
+    }
+    __syncthreads();
+    // the `keep` best groups, one after the other; a kept group's score becomes +inf as its mark
+    for (int it = 0; it < keep; ++it) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+      for (int g = lane; g < groups; g += TP_WAVE) {
+        const float v = group_l[g];
+        if (v != INFINITY && (v > bv || (v == bv && g < bi))) {
+          bv = v;
+          bi = g;
+        }
+      }
+      wave_arg_best(bv, bi);
+      __syncthreads();
+      if (lane == 0 && bi != 0x7fffffff) group_l[bi] = INFINITY;
+      __syncthreads();
+    }
+#pragma unroll
+    for (int k = 0; k < ROUTE_PER_LANE; ++k) {
+      const int e = lane + k * TP_WAVE;
+      if (e < experts && group_l[e / per] != INFINITY) ch[k] = -INFINITY;
+    }
+  }
+  for (int it = 0; it < top; ++it) {
+    float bv = -INFINITY, bs = 0.f;
+    int bi = 0x7fffffff, bk = -1;
+#pragma unroll
+    for (int k = 0; k < ROUTE_PER_LANE; ++k) {
+      const int e = lane + k * TP_WAVE;
+      if (e < experts && ch[k] > bv) {   // (ascending e within a lane: the lower index wins a tie)
+        bv = ch[k];
+        bi = e;
+        bk = k;
+        bs = sc[k];
+      }
+    }
+    float v = bv;
+    int i = bi;
+    wave_arg_best(v, i);
+    if (i == 0x7fffffff) break;   // fewer allowed experts than `top` (uniform over the wave)
+    if (i == bi && bk >= 0) {
+      // this lane owns the winner
+#pragma unroll
+      for (int k = 0; k < ROUTE_PER_LANE; ++k)
+        if (k == bk) ch[k] = -INFINITY;
+      if (live) {
+        dense[(size_t)t * experts + i] = bs;
+        ids[(size_t)t * top + it] = i;
+        weights[(size_t)t * top + it] = bs;
+      }
+    }
+  }
+}
+
+extern "C" int tp_moe_route(const float* logits, int logit_stride, const float* correction, int experts, int top, int groups,
+                            int keep, float* dense, int* ids, float* weights, int n, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && experts > 0 && top > 0 && top <= experts && logit_stride >= experts, "moe_route: bad sizes");
+  TP_REQUIRE(experts <= TP_WAVE * ROUTE_PER_LANE, "moe_route: %d experts exceed %d", experts, TP_WAVE * ROUTE_PER_LANE);
+  TP_REQUIRE(groups <= 1 || (experts % groups == 0 && keep >= 1 && keep <= groups), "moe_route: bad groups");
+  if (n == 0) return 0;
+  const size_t shmem = sizeof(float) * 4 * (size_t)(experts + (groups > 1 ? groups : 1));
+  hipLaunchKernelGGL(moe_route_kernel, dim3((n + 3) / 4), dim3(256), shmem, s, logits, logit_stride, correction, experts, top, groups,
+                     keep, dense, ids, weights, n);
+  TP_CHECK_LAUNCH("moe_route");
+  return 0;
+}
+
+// y[t] += dense[t, e] * part[t]: the weighted sum of the experts' outputs, one expert after the other.
+__global__ void moe_accumulate_kernel(float* __restrict__ y, const float* __restrict__ part, const float* __restrict__ dense,
+                                      int experts, int e, int width, size_t total, int first) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / width;
+  const float w = dense[t * experts + e];
+  y[i] = first ? w * part[i] : fmaf(w, part[i], y[i]);
+}
+
+extern "C" int tp_moe_accumulate(float* y, const float* part, const float* dense, int experts, int e, int n, int width, int first,
+                                 hipStream_t s) {
+  TP_REQUIRE(n >= 0 && width > 0 && e >= 0 && e < experts, "moe_accumulate: bad sizes");
+  if (n == 0) return 0;
+  const size_t total = (size_t)n * width;
+  hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, y, part, dense, experts, e,
+                     width, total, first);
+  TP_CHECK_LAUNCH("moe_accumulate");
+  return 0;
+}

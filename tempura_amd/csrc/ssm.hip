@@ -15,15 +15,16 @@ __device__ inline float silu_f(float v) { return v / (1.0f + expf(-v)); }
 // ln(1 + e^v) without overflow: max(v, 0) + ln(1 + e^-|v|)
 __device__ inline float softplus_f(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 
-// ---- causal convolution per channel + SiLU ----------------------------------------------------
+// ---- causal convolution per channel (+ SiLU) --------------------------------------------------
 // in: rows [n, in_stride] float32, the channels at column col0; w [taps, channels] (tap-major, so that the lanes of
-// a wave read neighbouring weights; the last tap is the current token's), b [channels].  The inputs before a run's first token come from the request's state row (zeros for a
-// fresh request).  out [n, channels] = silu(conv + b).
+// a wave read neighbouring weights; the last tap is the current token's), b [channels] or none.  The inputs before
+// a run's first token come from the request's state row, from element state_off on (zeros for a fresh request).
+// out [n, channels] = silu(conv + b), or conv + b itself when `act` is 0.
 __global__ void causal_conv_kernel(const float* __restrict__ in, int in_stride, int col0, const float* __restrict__ w,
                                    const float* __restrict__ b, const float* __restrict__ state, size_t state_stride,
                                    const int* __restrict__ cu_seqlens, const int* __restrict__ token_req,
                                    const int* __restrict__ state_slots, float* __restrict__ out, int channels, int taps,
-                                   int channel_blocks) {
+                                   int channel_blocks, size_t state_off, int act) {
   // (neighbouring blocks take neighbouring channels of one token: they read one row of the input after the other)
   const int t = blockIdx.x / channel_blocks;
   const int c = (blockIdx.x % channel_blocks) * blockDim.x + threadIdx.x;
@@ -31,27 +32,27 @@ __global__ void causal_conv_kernel(const float* __restrict__ in, int in_stride, 
   const int r = token_req[t];
   const int start = cu_seqlens[r];
   const int i = t - start;
-  const float* st = state + (size_t)state_slots[r] * state_stride;
-  float acc = b[c];
+  const float* st = state + (size_t)state_slots[r] * state_stride + state_off;
+  float acc = b != nullptr ? b[c] : 0.f;
   for (int k = 0; k < taps; ++k) {
     const int src = i - (taps - 1 - k);
     const float v = src >= 0 ? in[(size_t)(start + src) * in_stride + col0 + c] : st[(size_t)(taps - 1 + src) * channels + c];
     acc = fmaf(w[(size_t)k * channels + c], v, acc);
   }
-  out[(size_t)t * channels + c] = silu_f(acc);
+  out[(size_t)t * channels + c] = act ? silu_f(acc) : acc;
 }
 
 // The state after a run: the last taps - 1 inputs of (carried inputs, then the run's).  In place, ascending: entry j
 // takes entry j + len of the old state or an input of the run, and entries below j are never read again.
 __global__ void conv_state_kernel(const float* __restrict__ in, int in_stride, int col0, float* __restrict__ state,
                                   size_t state_stride, const int* __restrict__ cu_seqlens,
-                                  const int* __restrict__ state_slots, int channels, int taps) {
+                                  const int* __restrict__ state_slots, int channels, int taps, size_t state_off) {
   const int r = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= channels) return;
   const int start = cu_seqlens[r], len = cu_seqlens[r + 1] - start;
   if (len <= 0) return;
-  float* st = state + (size_t)state_slots[r] * state_stride;
+  float* st = state + (size_t)state_slots[r] * state_stride + state_off;
   for (int j = 0; j < taps - 1; ++j) {
     const int src = len - (taps - 1) + j;
     const float v = src >= 0 ? in[(size_t)(start + src) * in_stride + col0 + c] : st[(size_t)(j + len) * channels + c];
@@ -60,19 +61,20 @@ __global__ void conv_state_kernel(const float* __restrict__ in, int in_stride, i
 }
 
 extern "C" int tp_causal_conv(const float* in, int in_stride, int col0, const float* w, const float* b, float* state,
-                              size_t state_stride, const int* cu_seqlens, const int* token_req, const int* state_slots,
-                              float* out, int n, int n_req, int channels, int taps, hipStream_t s) {
+                              size_t state_stride, size_t state_off, const int* cu_seqlens, const int* token_req,
+                              const int* state_slots, float* out, int n, int n_req, int channels, int taps, int act,
+                              hipStream_t s) {
   TP_REQUIRE(n >= 0 && n_req >= 0 && channels > 0 && taps >= 1, "causal_conv: bad sizes");
-  TP_REQUIRE(in_stride >= col0 + channels && state_stride >= (size_t)(taps - 1) * channels, "causal_conv: rows too short");
+  TP_REQUIRE(in_stride >= col0 + channels && state_stride >= state_off + (size_t)(taps - 1) * channels, "causal_conv: rows too short");
   if (n == 0) return 0;
   const int threads = channels >= 256 ? 256 : 64;
   const int cb = (channels + threads - 1) / threads;
   TP_REQUIRE(cb <= 65535 && (long)n * cb < 0x7fffffffL, "causal_conv: too many channels or tokens");
   hipLaunchKernelGGL(causal_conv_kernel, dim3((unsigned)((long)n * cb)), dim3(threads), 0, s, in, in_stride, col0, w, b, state,
-                     state_stride, cu_seqlens, token_req, state_slots, out, channels, taps, cb);
+                     state_stride, cu_seqlens, token_req, state_slots, out, channels, taps, cb, state_off, act);
   if (taps > 1 && n_req > 0)
     hipLaunchKernelGGL(conv_state_kernel, dim3(n_req, cb), dim3(threads), 0, s, in, in_stride, col0, state,
-                       state_stride, cu_seqlens, state_slots, channels, taps);
+                       state_stride, cu_seqlens, state_slots, channels, taps, state_off);
   TP_CHECK_LAUNCH("causal_conv");
   return 0;
 }

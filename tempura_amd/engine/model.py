@@ -20,6 +20,9 @@ from ..parts.inventory import expected_weights
 
 
 class CausalLM:
+    #: key of the embedding's per-request state among the state tensors (the others are cache slot numbers)
+    EMBEDDING_STATE = -1
+
     def __init__(self, spec: ModelSpec, dtype: torch.dtype, device):
         if dtype not in (torch.bfloat16, torch.float32):
             raise ValueError(f"compute dtype must be bfloat16 or float32, got {dtype}")
@@ -76,6 +79,10 @@ class CausalLM:
             if ss is not None:
                 self.state_specs[slot] = ss
         self.slots_per_group = counts
+        #: per-request state that belongs to the model's ends rather than to a layer: key -1 of the state tensors
+        es = self.embedding.state_spec() if hasattr(self.embedding, "state_spec") else None
+        if es is not None:
+            self.state_specs[self.EMBEDDING_STATE] = es
         for i, call in enumerate(self.order):
             if not self.call_writes[i]:
                 mine = self._cache_owner(call.layer).cache_spec()
@@ -125,12 +132,17 @@ class CausalLM:
         return total
 
     # ---- forward -------------------------------------------------------
-    def forward(self, tokens: torch.Tensor, ctx, caches) -> torch.Tensor:
-        """``tokens`` int32 [n]; ``caches[i]`` is the ``LayerCache`` of run-order entry i.
+    def forward(self, tokens: torch.Tensor, ctx, caches, state=None) -> torch.Tensor:
+        """``tokens`` int32 [n]; ``caches[i]`` is the ``LayerCache`` of run-order entry i; ``state``: the state
+        tensors by key, for the per-request state of the model's ends (``EMBEDDING_STATE``).
         Returns float32 logits [len(ctx.logit_rows), vocab]."""
         if hasattr(ctx, "shared"):
             ctx.shared.clear()      # what layers share is computed anew in every pass (also in one that is captured)
-        if self.streams > 1 or getattr(self.embedding, "inv_freq", None) is not None:
+        if self.EMBEDDING_STATE in self.state_specs:
+            if state is None or self.EMBEDDING_STATE not in state:
+                raise ValueError("this model's embedding keeps per-request state: forward needs the state tensors")
+            h = self.embedding.forward(tokens, ctx.positions, self.streams, ctx=ctx, state=state[self.EMBEDDING_STATE])
+        elif self.streams > 1 or getattr(self.embedding, "inv_freq", None) is not None:
             h = self.embedding.forward(tokens, ctx.positions, self.streams)
         else:
             h = self.embedding.forward(tokens)

@@ -392,13 +392,13 @@ class ModelRunner:
             # one eager run first: lazy initialisation must not happen under capture.  (What it writes into the
             # paged cache the replay writes again; per-request state it would advance twice, so that is put back.)
             kept = {slot: t.clone() for slot, t in self.pools.state.items()}
-            self.model.forward(tok, ctx, self.layer_caches)
+            self.model.forward(tok, ctx, self.layer_caches, self.pools.state)
             for slot, t in kept.items():
                 self.pools.state[slot].copy_(t)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self._graph_pool):
-                g.logits = self.model.forward(tok, ctx, self.layer_caches)
+                g.logits = self.model.forward(tok, ctx, self.layer_caches, self.pools.state)
             if self._graph_pool is None:
                 self._graph_pool = graph.pool()
             g.graph = graph
@@ -460,7 +460,7 @@ class ModelRunner:
         tok_dev, ctx = self._pack_step(entries)
         if self.pools.state:
             self._clear_state([s for s, n, c in zip(ctx.state_slot_list, ctx.q_lens, ctx.ctx_lens) if c == n])
-        logits = self.model.forward(tok_dev, ctx, self.layer_caches)
+        logits = self.model.forward(tok_dev, ctx, self.layer_caches, self.pools.state)
         self.cache.commit_many([e.rid for e in entries], ctx.q_lens)
         self.steps_run += 1
         self.tokens_run += ctx.num_tokens

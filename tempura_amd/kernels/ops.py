@@ -283,29 +283,35 @@ def qk_store(rows: torch.Tensor, q_bias: Optional[torch.Tensor], k_bias: Optiona
     return q
 
 
-def causal_conv(proj: torch.Tensor, col0: int, channels: int, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor,
-                cu_seqlens: torch.Tensor, token_req: torch.Tensor, state_slots: torch.Tensor, num_requests: int) -> torch.Tensor:
-    """Causal convolution per channel over each request's run of tokens, then SiLU.  ``proj`` float32 [n, width]
-    holds the inputs at columns col0 .. col0 + channels; ``weight`` [taps, channels] (tap-major; the last tap is the
-    current token's), ``bias`` [channels]; ``state`` float32 [slots, row] whose rows start with the carried inputs
-    [taps - 1, channels] (oldest first) of the request in that slot: they are read for the first tokens of a run
-    and replaced by the run's last inputs.  Returns float32 [n, channels]."""
+def causal_conv(proj: torch.Tensor, col0: int, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+                cu_seqlens: torch.Tensor, token_req: torch.Tensor, state_slots: torch.Tensor, num_requests: int,
+                state_off: int = 0, act: bool = True) -> torch.Tensor:
+    """Causal convolution per channel over each request's run of tokens, then SiLU (``act`` False: the sums
+    themselves).  ``proj`` float32 [n, width] holds the inputs at columns col0 .. col0 + channels; ``weight``
+    [taps, channels] (tap-major; the last tap is the current token's), ``bias`` [channels] or None; ``state`` float32
+    [slots, row] whose rows hold, from element ``state_off`` on, the carried inputs [taps - 1, channels] (oldest
+    first) of the request in that slot: they are read for the first tokens of a run and replaced by the run's last
+    inputs.  Returns float32 [n, channels]."""
     if _backend is not None:
-        return _backend.causal_conv(proj, col0, channels, weight, bias, state, cu_seqlens, token_req, state_slots, num_requests)
+        if state_off == 0 and act and bias is not None:
+            return _backend.causal_conv(proj, col0, channels, weight, bias, state, cu_seqlens, token_req, state_slots, num_requests)
+        return _backend.causal_conv(proj, col0, channels, weight, bias, state, cu_seqlens, token_req, state_slots, num_requests,
+                                    state_off, act)
     _dev_ok(proj, weight, bias, state, cu_seqlens, token_req, state_slots)
     _need(proj.dtype == torch.float32 and proj.dim() == 2 and 0 <= col0 and col0 + channels <= proj.shape[1], "causal_conv: bad rows")
     _need(weight.dtype == torch.float32 and weight.dim() == 2 and weight.shape[1] == channels, "causal_conv: weight must be float32 [taps, channels]")
     taps = weight.shape[0]
-    _need(bias.dtype == torch.float32 and bias.numel() == channels, "causal_conv: bias must be float32 [channels]")
-    _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= (taps - 1) * channels, "causal_conv: state rows too short")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == channels), "causal_conv: bias must be float32 [channels]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state_off >= 0 and state.shape[1] >= state_off + (taps - 1) * channels,
+          "causal_conv: state rows too short")
     n = proj.shape[0]
     _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
     _i32(state_slots, num_requests, "state_slots")
     _i32(token_req, n, "token_req") if n else None
     out = torch.empty((n, channels), dtype=torch.float32, device=proj.device)
     _call("tp_causal_conv", _ptr(proj), proj.shape[1], int(col0), _ptr(weight), _ptr(bias), _ptr(state),
-          ctypes.c_size_t(state.shape[1]), _ptr(cu_seqlens), _ptr(token_req), _ptr(state_slots), _ptr(out), n, int(num_requests),
-          channels, taps, _stream())
+          ctypes.c_size_t(state.shape[1]), ctypes.c_size_t(state_off), _ptr(cu_seqlens), _ptr(token_req), _ptr(state_slots), _ptr(out),
+          n, int(num_requests), channels, taps, int(bool(act)), _stream())
     return out
 
 
@@ -728,14 +734,20 @@ def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
                   inv_freq: Optional[torch.Tensor], rotary_dim: int, factor: float, num_heads: int,
                   num_kv_heads: int, head_dim: int, k_cache: Optional[torch.Tensor],
                   v_cache: Optional[torch.Tensor], q_dtype: torch.dtype,
-                  cos_sin: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  cos_sin: Optional[torch.Tensor] = None, value_dim: Optional[int] = None) -> torch.Tensor:
     """Rotate q and k of float32 rows [n, (heads + 2 kv_heads) * head_dim] (or the ``Partials`` of the
     projection that makes them), store k and v into the cache rows ``slots`` and return q as q_dtype
     [n, heads, head_dim].  With ``slots`` None the rows hold q only and nothing is stored.
+    ``value_dim``: the size of a value head when it is not head_dim (the rows are then
+    [n, (heads + kv_heads) * head_dim + kv_heads * value_dim], the value cache [pages, kv_heads, value_dim, page_size]).
     The q and k heads are in PAIRED order: elements (2 d, 2 d + 1) of a head rotate together by the angle
     of pair d (they are elements (d, d + rotary_dim / 2) of the split-half order).
     ``cos_sin``: this step's table from ``rope_table`` (the same values, computed once for all layers)."""
+    vd = head_dim if value_dim is None else int(value_dim)
     if _backend is not None:
+        if vd != head_dim:
+            return _backend.rope_kv_write(qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads,
+                                          num_kv_heads, head_dim, k_cache, v_cache, q_dtype, value_dim=vd)
         return _backend.rope_kv_write(qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads,
                                       num_kv_heads, head_dim, k_cache, v_cache, q_dtype)
     splits = 1
@@ -746,15 +758,15 @@ def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
     _need(qkv.is_cuda, "operand is not on the GPU")
     _need(qkv.dtype == torch.float32 and qkv.dim() == 2, "rope_kv_write: rows must be float32 [n, width]")
     n = qkv.shape[0]
-    width = (num_heads + (2 * num_kv_heads if slots is not None else 0)) * head_dim
+    width = (num_heads + (num_kv_heads if slots is not None else 0)) * head_dim + (num_kv_heads * vd if slots is not None else 0)
     _need(qkv.shape[1] == width, f"rope_kv_write: row width {qkv.shape[1]} != {width}")
     _i32(positions, n, "positions") if n else None
     page_size, cache_dt = 1, _F32
     if slots is not None:
         _i32(slots, n, "slots") if n else None
         _need(k_cache is not None and v_cache is not None and k_cache.dim() == 4 and v_cache.dim() == 4
-              and tuple(v_cache.shape) == (k_cache.shape[0], k_cache.shape[1], k_cache.shape[3], k_cache.shape[2]),
-              "rope_kv_write: caches must be k [pages, kv_heads, page_size, head_dim], v [pages, kv_heads, head_dim, page_size]")
+              and tuple(v_cache.shape) == (k_cache.shape[0], k_cache.shape[1], vd, k_cache.shape[2]),
+              "rope_kv_write: caches must be k [pages, kv_heads, page_size, head_dim], v [pages, kv_heads, value_dim, page_size]")
         _need(k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == head_dim, "rope_kv_write: cache layout mismatch")
         _need(k_cache.dtype == v_cache.dtype, "rope_kv_write: cache dtypes differ")
         page_size, cache_dt = k_cache.shape[2], _dt(k_cache)
@@ -767,7 +779,7 @@ def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
     q = torch.empty((n, num_heads, head_dim), dtype=q_dtype, device=qkv.device)
     _call("tp_rope_kv_write", _ptr(qkv), qkv.shape[1], _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
           ctypes.c_float(factor), n, num_heads, num_kv_heads, head_dim, _ptr(q), _dtcode(q_dtype),
-          _ptr(k_cache), _ptr(v_cache), cache_dt, page_size, splits, _ptr(cos_sin), _stream())
+          _ptr(k_cache), _ptr(v_cache), cache_dt, page_size, splits, _ptr(cos_sin), vd, _stream())
     return q
 
 
@@ -819,7 +831,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     scale: float, window: int, max_q_len: int, max_context_len: int,
                     num_single: Optional[int] = None, dist_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [n, heads, head_dim] over k [pages, kv_heads, page_size, head_dim] and transposed
-    v [pages, kv_heads, head_dim, page_size] -> [n, heads * head_dim].
+    v [pages, kv_heads, value_dim, page_size] -> [n, heads * value_dim] (value_dim is the value cache's own; the
+    matrix-core kernels take value_dim == head_dim, other sizes run the general kernel).
     ``dist_bias`` (float32 [heads, L]): added to the scaled score of a query at position p and a key at j as
     dist_bias[head, min(p - j, L - 1)]."""
     if _backend is not None:
@@ -834,7 +847,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _need(q.dim() == 3 and k_cache.dim() == 4 and v_cache.dim() == 4, "paged_attention: bad operand ranks")
     n, heads, d = q.shape
     pages, kvh, page_size, d2 = k_cache.shape
-    _need(tuple(v_cache.shape) == (pages, kvh, d2, page_size), "paged_attention: v cache must be [pages, kv_heads, head_dim, page_size]")
+    vd = v_cache.shape[2]
+    _need(tuple(v_cache.shape) == (pages, kvh, vd, page_size), "paged_attention: v cache must be [pages, kv_heads, value_dim, page_size]")
     _need(d == d2, "paged_attention: head_dim of q and cache differ")
     _need(q.dtype == k_cache.dtype == v_cache.dtype, "paged_attention: q and cache dtypes differ")
     _need(block_tables.dim() == 2 and block_tables.dtype == torch.int32, "paged_attention: block_tables must be int32 [r, width]")
@@ -844,7 +858,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _i32(token_req, n, "token_req") if n else None
     _need(pages * kvh * page_size < 2 ** 31, "paged_attention: cache pool too large for 32-bit row indices")
     _need(max_context_len <= width * page_size, "paged_attention: block table narrower than the longest context")
-    out = torch.empty((n, heads * d), dtype=q.dtype, device=q.device)
+    out = torch.empty((n, heads * vd), dtype=q.dtype, device=q.device)
     if num_single is None:
         num_single = r if max_q_len == 1 else 0
     _need(0 <= num_single <= r, "paged_attention: num_single out of range")
@@ -852,7 +866,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _dev_ok(dist_bias)
         _need(dist_bias.dtype == torch.float32 and dist_bias.dim() == 2 and dist_bias.shape[0] == heads and dist_bias.shape[1] > 0,
               "paged_attention: dist_bias must be float32 [heads, L]")
-    fast = allow_fast_attention and q.dtype == torch.bfloat16 and d % 32 == 0 and d <= 128 and page_size % 8 == 0
+    fast = allow_fast_attention and q.dtype == torch.bfloat16 and d % 32 == 0 and d <= 128 and page_size % 8 == 0 and vd == d
     splits, scratch = 1, None
     if fast and num_single > 0:
         # enough blocks to fill 256 CUs, but at least 128 keys per block
@@ -902,7 +916,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
           _ptr(cu_seqlens), _ptr(context_lens), _ptr(token_req), _ptr(out), n, r, heads, kvh, d, page_size,
           ctypes.c_float(scale), int(window), int(max_q_len), int(max_context_len), int(fast),
           int(num_single), int(splits), _ptr(scratch), int(parts), max(1, portion_min_keys // 32), _ptr(part_scratch),
-          _ptr(dist_bias), 0 if dist_bias is None else dist_bias.shape[1], _stream())
+          _ptr(dist_bias), 0 if dist_bias is None else dist_bias.shape[1], int(vd), _stream())
     return out
 
 
@@ -1160,3 +1174,189 @@ def fill_normal(out: torch.Tensor, seed: int, mean: float, std: float) -> torch.
     _call("tp_fill_normal", _ptr(out), _dt(out), ctypes.c_size_t(out.numel()), ctypes.c_ulonglong(seed & (2 ** 64 - 1)),
           ctypes.c_double(mean), ctypes.c_double(std), _stream())
     return out
+
+
+# ---------------------------------------------------------------------------------
+# Operations of layers with a hashed bigram embedding, norms behind the sublayers, a gated delta-rule mixer and
+# routed experts.
+
+def embed_bigram(tokens: torch.Tensor, table: torch.Tensor, bigram: torch.Tensor, positions: torch.Tensor,
+                 token_req: torch.Tensor, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, prev_state: torch.Tensor,
+                 num_requests: int, mul_prev: int, mul_cur: int, buckets: int) -> torch.Tensor:
+    """float32 [n, hidden] = table[token] + bigram[row], row = (previous * mul_prev + token * mul_cur) mod buckets,
+    and row ``buckets`` for a token at position 0.  The previous token of a run's first token is what
+    ``prev_state`` (int32 [slots, 1]) holds for the request's slot; each run's last token is left there."""
+    if _backend is not None:
+        return _backend.embed_bigram(tokens, table, bigram, positions, token_req, cu_seqlens, state_slots, prev_state,
+                                     num_requests, mul_prev, mul_cur, buckets)
+    _dev_ok(tokens, table, bigram, positions, token_req, cu_seqlens, state_slots, prev_state)
+    n = tokens.numel()
+    _need(table.dim() == 2 and bigram.dim() == 2 and bigram.shape[1] == table.shape[1] and bigram.dtype == table.dtype,
+          "embed_bigram: tables must be [rows, hidden] of one type")
+    _need(bigram.shape[0] == buckets + 1, f"embed_bigram: the bigram table needs {buckets + 1} rows, has {bigram.shape[0]}")
+    _i32(tokens, n, "embed tokens") if n else None
+    _i32(positions, n, "embed positions") if n else None
+    _i32(token_req, n, "token_req") if n else None
+    _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
+    _i32(state_slots, num_requests, "state_slots")
+    _need(prev_state.dtype == torch.int32, "embed_bigram: the state must be int32")
+    hidden = table.shape[1]
+    out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
+    _call("tp_embed_bigram", _ptr(tokens), _ptr(positions), _ptr(token_req), _ptr(cu_seqlens), _ptr(state_slots), _ptr(prev_state),
+          _ptr(table), _ptr(bigram), _dt(table), _ptr(out), n, int(num_requests), hidden, ctypes.c_longlong(mul_prev),
+          ctypes.c_longlong(mul_cur), ctypes.c_longlong(buckets), _stream())
+    return out
+
+
+def sigmoid_gate(a: torch.Tensor, proj: Optional[torch.Tensor], gate_col0: int, scale: float, out: torch.Tensor, out_col0: int) -> None:
+    """out[:, out_col0 + c] = a[:, c] * sigmoid(proj[:, gate_col0 + c]) * scale (``proj`` float32 rows; None: no
+    gate); ``a`` and ``out`` are of one type, ``out`` [n, wider]."""
+    if _backend is not None:
+        return _backend.sigmoid_gate(a, proj, gate_col0, scale, out, out_col0)
+    _dev_ok(a, proj, out)
+    _need(a.dim() == 2 and out.dim() == 2 and a.dtype == out.dtype and a.shape[0] == out.shape[0], "sigmoid_gate: bad operands")
+    n, width = a.shape
+    _need(0 <= out_col0 and out_col0 + width <= out.shape[1], "sigmoid_gate: output rows too short")
+    if proj is not None:
+        _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.shape[0] == n and 0 <= gate_col0 and gate_col0 + width <= proj.shape[1],
+              "sigmoid_gate: bad gate rows")
+    _call("tp_sigmoid_gate", _ptr(a), _dt(a), _ptr(proj), 0 if proj is None else proj.shape[1], int(gate_col0), ctypes.c_float(scale),
+          _ptr(out), out.shape[1], int(out_col0), n, width, _stream())
+
+
+def norm_add(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, next_weight: Optional[torch.Tensor] = None,
+             next_eps: float = 0.0, out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """h += y / sqrt(mean(y^2) + eps) * weight, per row, in place (float32 [n, width]).  With ``next_weight`` the
+    rows of the new h normed with it (and ``next_eps``) come back as ``out_dtype``."""
+    if _backend is not None:
+        return _backend.norm_add(h, y, weight, eps, next_weight, next_eps, out_dtype)
+    _dev_ok(h, y, weight, next_weight)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and y.dtype == torch.float32 and tuple(y.shape) == tuple(h.shape),
+          "norm_add: h and y must be float32 [n, width]")
+    n, width = h.shape
+    _need(weight.dtype == torch.float32 and weight.numel() == width, "norm_add: weight must be float32 [width]")
+    x = None
+    if next_weight is not None:
+        _need(next_weight.dtype == torch.float32 and next_weight.numel() == width and out_dtype is not None, "norm_add: bad next norm")
+        x = torch.empty((n, width), dtype=out_dtype, device=h.device)
+    _call("tp_norm_add", _ptr(h), _ptr(y), _ptr(weight), ctypes.c_float(eps), _ptr(next_weight), ctypes.c_float(next_eps), _ptr(x),
+          _dtcode(out_dtype) if x is not None else _F32, n, width, _stream())
+    return x
+
+
+ACTIVATIONS = {"gelu_tanh": 0, "silu": 1}
+
+
+def activation(u: torch.Tensor, kind: str, out_dtype: torch.dtype) -> torch.Tensor:
+    """Element by element: ``gelu_tanh`` (0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))) or ``silu``, formed in
+    float32, as ``out_dtype``."""
+    _need(kind in ACTIVATIONS, f"activation: {kind!r} unknown (known: {sorted(ACTIVATIONS)})")
+    if _backend is not None:
+        return _backend.activation(u, kind, out_dtype)
+    _dev_ok(u)
+    out = torch.empty(u.shape, dtype=out_dtype, device=u.device)
+    _call("tp_activation", _ptr(u), _dt(u), _ptr(out), _dtcode(out_dtype), ctypes.c_size_t(u.numel()), ACTIVATIONS[kind], _stream())
+    return out
+
+
+def moe_route(logits: torch.Tensor, correction: torch.Tensor, experts: int, top: int, groups: int, keep: int):
+    """Router of a mixture of experts over float32 logits [n, >= experts]: s = softmax over the experts; an expert's
+    choice score is s + correction; with ``groups`` > 1 only the experts of the ``keep`` groups (of neighbours) with
+    the largest best choice score can be chosen; the ``top`` best allowed experts are chosen and weigh s.  Returns
+    (dense float32 [n, experts] with a chosen expert's weight and 0 elsewhere, ids int32 [n, top], weights [n, top])."""
+    if _backend is not None:
+        return _backend.moe_route(logits, correction, experts, top, groups, keep)
+    _dev_ok(logits, correction)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[1] >= experts, "moe_route: logits must be float32 [n, experts]")
+    _need(correction.dtype == torch.float32 and correction.numel() == experts, "moe_route: correction must be float32 [experts]")
+    n = logits.shape[0]
+    dense = torch.empty((n, experts), dtype=torch.float32, device=logits.device)
+    ids = torch.empty((n, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((n, top), dtype=torch.float32, device=logits.device)
+    _call("tp_moe_route", _ptr(logits), logits.shape[1], _ptr(correction), int(experts), int(top), int(groups), int(keep), _ptr(dense),
+          _ptr(ids), _ptr(weights), n, _stream())
+    return dense, ids, weights
+
+
+def moe_accumulate(y: Optional[torch.Tensor], part: torch.Tensor, dense: torch.Tensor, expert: int) -> torch.Tensor:
+    """y[t] += dense[t, expert] * part[t] (float32 [n, width]); ``y`` None: a new tensor holding the product."""
+    if _backend is not None:
+        return _backend.moe_accumulate(y, part, dense, expert)
+    _dev_ok(y, part, dense)
+    _need(part.dtype == torch.float32 and part.dim() == 2 and dense.dtype == torch.float32 and dense.dim() == 2
+          and dense.shape[0] == part.shape[0] and 0 <= expert < dense.shape[1], "moe_accumulate: bad operands")
+    first = y is None
+    if first:
+        y = torch.empty_like(part)
+    _need(y.dtype == torch.float32 and tuple(y.shape) == tuple(part.shape), "moe_accumulate: y must match the expert's output")
+    _call("tp_moe_accumulate", _ptr(y), _ptr(part), _ptr(dense), dense.shape[1], int(expert), part.shape[0], part.shape[1], int(first),
+          _stream())
+    return y
+
+
+LOWRANK_MODES = {"plain": 0, "sigmoid": 1, "decay": 2}
+
+
+def lowrank_up(x: torch.Tensor, col0: int, weight_t: torch.Tensor, mode: str = "plain", a_log: Optional[torch.Tensor] = None,
+               bias: Optional[torch.Tensor] = None, per_head: int = 0) -> torch.Tensor:
+    """The second product of a low-rank projection: float32 [n, N] = f(x[:, col0: col0 + r] @ weight_t), ``x`` float32
+    rows (the first product's sums), ``weight_t`` float32 [r, N].  f: ``plain``; ``sigmoid``; ``decay``:
+    exp(-exp(a_log[c // per_head]) * softplus(sum + bias[c]))."""
+    if _backend is not None:
+        return _backend.lowrank_up(x, col0, weight_t, mode, a_log, bias, per_head)
+    _dev_ok(x, weight_t, a_log, bias)
+    _need(mode in LOWRANK_MODES, f"lowrank_up: mode {mode!r} unknown")
+    _need(x.dtype == torch.float32 and x.dim() == 2 and weight_t.dtype == torch.float32 and weight_t.dim() == 2, "lowrank_up: float32 operands")
+    r, n_out = weight_t.shape
+    _need(0 <= col0 and col0 + r <= x.shape[1], "lowrank_up: rows too short")
+    if mode == "decay":
+        _need(a_log is not None and bias is not None and per_head > 0 and n_out % per_head == 0 and a_log.dtype == torch.float32
+              and bias.dtype == torch.float32 and a_log.numel() == n_out // per_head and bias.numel() == n_out, "lowrank_up: bad decay constants")
+    out = torch.empty((x.shape[0], n_out), dtype=torch.float32, device=x.device)
+    _call("tp_lowrank_up", _ptr(x), x.shape[1], int(col0), r, _ptr(weight_t), _ptr(out), x.shape[0], n_out, LOWRANK_MODES[mode],
+          _ptr(a_log), _ptr(bias), int(per_head), _stream())
+    return out
+
+
+def delta_scan(qkv: torch.Tensor, decay: torch.Tensor, proj: torch.Tensor, beta_col0: int, state: torch.Tensor, state_off: int,
+               cu_seqlens: torch.Tensor, state_slots: torch.Tensor, num_requests: int, heads: int, kv_heads: int, dim: int,
+               vdim: int, q_scale: float, unit_eps: float) -> torch.Tensor:
+    """The gated delta rule per head over each request's run.  ``qkv`` float32 [n, q | k | v] with q and k
+    [kv_heads * dim] and v [heads * vdim]; q and k are made unit vectors per head (x / sqrt(sum x^2 + unit_eps), q times
+    ``q_scale``); beta = sigmoid(proj[:, beta_col0 + h]); ``decay`` float32 [n, heads * dim].  Per head, with S
+    [dim, vdim] at ``state[slot, state_off:]``:  S <- decay * S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
+    Returns o float32 [n, heads * vdim]; the state is left as the run leaves it."""
+    if _backend is not None:
+        return _backend.delta_scan(qkv, decay, proj, beta_col0, state, state_off, cu_seqlens, state_slots, num_requests, heads,
+                                   kv_heads, dim, vdim, q_scale, unit_eps)
+    _dev_ok(qkv, decay, proj, state, cu_seqlens, state_slots)
+    n = qkv.shape[0]
+    _need(qkv.dtype == torch.float32 and qkv.dim() == 2 and qkv.shape[1] == 2 * kv_heads * dim + heads * vdim, "delta_scan: bad q | k | v rows")
+    _need(decay.dtype == torch.float32 and tuple(decay.shape) == (n, heads * dim), "delta_scan: decay must be float32 [n, heads * dim]")
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.shape[0] == n and 0 <= beta_col0 and beta_col0 + heads <= proj.shape[1],
+          "delta_scan: bad projection rows")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state_off >= 0 and state.shape[1] >= state_off + heads * dim * vdim,
+          "delta_scan: state rows too short")
+    _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
+    _i32(state_slots, num_requests, "state_slots")
+    y = torch.empty((n, heads * vdim), dtype=torch.float32, device=qkv.device)
+    _call("tp_delta_scan", _ptr(qkv), qkv.shape[1], _ptr(decay), _ptr(proj), proj.shape[1], int(beta_col0), _ptr(state),
+          ctypes.c_size_t(state.shape[1]), ctypes.c_size_t(state_off), _ptr(cu_seqlens), _ptr(state_slots), _ptr(y), int(num_requests),
+          int(heads), int(kv_heads), int(dim), int(vdim), ctypes.c_float(q_scale), ctypes.c_float(unit_eps), _stream())
+    return y
+
+
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.Tensor], eps: float, scale: float, heads: int,
+                   out: torch.Tensor, out_col0: int) -> None:
+    """out[:, out_col0 + h * vdim + d] = o[:, h, d] / sqrt(mean_d o^2 + eps) * weight[d] * gate[:, h * vdim + d] * scale:
+    ``o`` float32 [n, heads * vdim], ``weight`` float32 [vdim] shared by the heads, ``gate`` float32 like ``o`` or None."""
+    if _backend is not None:
+        return _backend.head_norm_gate(o, weight, gate, eps, scale, heads, out, out_col0)
+    _dev_ok(o, weight, gate, out)
+    _need(o.dtype == torch.float32 and o.dim() == 2 and o.shape[1] % heads == 0, "head_norm_gate: o must be float32 [n, heads * vdim]")
+    n, vdim = o.shape[0], o.shape[1] // heads
+    _need(weight.dtype == torch.float32 and weight.numel() == vdim, "head_norm_gate: weight must be float32 [vdim]")
+    _need(gate is None or (gate.dtype == torch.float32 and tuple(gate.shape) == tuple(o.shape)), "head_norm_gate: gate must match o")
+    _need(out.dim() == 2 and out.shape[0] == n and 0 <= out_col0 and out_col0 + o.shape[1] <= out.shape[1], "head_norm_gate: output rows too short")
+    _call("tp_head_norm_gate", _ptr(o), _ptr(weight), _ptr(gate), ctypes.c_float(eps), ctypes.c_float(scale), _ptr(out), _dt(out),
+          out.shape[1], int(out_col0), n, int(heads), vdim, _stream())

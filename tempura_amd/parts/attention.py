@@ -21,11 +21,12 @@ The first two need a position encoding that does not rotate (``"none"``).
 from __future__ import annotations
 
 import math
+from dataclasses import dataclass
 
 import torch
 
 from ..kernels import ops
-from .base import CacheSpec, Mixer, WeightInfo, build_part, part_class, register_part
+from .base import BranchMixer, CacheSpec, Mixer, WeightInfo, build_part, part_class, register_part
 
 
 def log_bucket(n: int, buckets: int, max_distance: int) -> int:
@@ -221,3 +222,115 @@ class PagedAttention(Mixer):
 
 
 register_part("mixer", "attention", PagedAttention)
+
+
+@dataclass(frozen=True)
+class SizedValueCacheSpec(CacheSpec):
+    """Keys of ``head_dim`` and values of ``value_dim``: keys [kv_heads, page_size, head_dim] as ever, values
+    transposed [kv_heads, value_dim, page_size]."""
+    value_dim: int = 0
+
+    def planes(self, page_size: int):
+        return {"k": (self.num_kv_heads, page_size, self.head_dim), "v": (self.num_kv_heads, self.value_dim, page_size)}
+
+
+class ConvAttention(BranchMixer):
+    """Grouped-query softmax attention over the paged cache whose q, k and v pass a short causal convolution per
+    channel right behind their projections (``conv_taps`` taps, no bias, no activation, zeros before a request's
+    start; before any rotation), whose values may have another size than its keys (``value_dim``), and whose
+    concatenated heads are multiplied by sigmoid(W_g x) before the output projection (``gate``).  The position
+    encoding, the scale and an optional window are parameters as for ``attention``.
+
+    The columns of its input product are [q | k | v | gate]; a request's state is the convolution's last
+    ``conv_taps - 1`` inputs [conv_taps - 1, q | k | v], float32."""
+    preferred_portion_align = 8      # (the value cache is transposed: see ``PagedAttention``)
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        p = spec.params
+        self.num_heads = int(p["num_heads"])
+        self.num_kv_heads = int(p["num_kv_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.value_dim = int(p.get("value_dim") or self.head_dim)
+        if self.num_heads % self.num_kv_heads != 0:
+            raise ValueError("conv_attention: heads must be a multiple of kv heads")
+        self.scale = float(p["scale"])
+        self.window = p.get("window")
+        self.taps = int(p["conv_taps"])
+        if self.taps < 1:
+            raise ValueError("conv_attention: conv_taps must be at least 1")
+        self.gate = bool(p.get("gate", False))
+        self.position = build_part("position", p["position"], hidden_size, dtype, device)
+        self.q_dim = self.num_heads * self.head_dim
+        self.k_dim = self.num_kv_heads * self.head_dim
+        self.v_dim = self.num_kv_heads * self.value_dim
+        self.channels = self.q_dim + self.k_dim + self.v_dim
+        self.inner = self.num_heads * self.value_dim
+        self.conv_w = None
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        p, w = spec.params, spec.weights
+        vd = int(p.get("value_dim") or p["head_dim"])
+        q_dim, k_dim, v_dim = p["num_heads"] * p["head_dim"], p["num_kv_heads"] * p["head_dim"], p["num_kv_heads"] * vd
+        taps = int(p["conv_taps"])
+        out = {
+            w["q"]: WeightInfo((q_dim, hidden_size)), w["k"]: WeightInfo((k_dim, hidden_size)), w["v"]: WeightInfo((v_dim, hidden_size)),
+            w["q_conv"]: WeightInfo((q_dim, taps)), w["k_conv"]: WeightInfo((k_dim, taps)),
+            w["v_conv"]: WeightInfo((v_dim, taps)),
+            w["o"]: WeightInfo((hidden_size, p["num_heads"] * vd)),
+        }
+        if p.get("gate", False):
+            out[w["gate"]] = WeightInfo((p["num_heads"] * vd, hidden_size))
+        out.update(part_class("position", p["position"].kind).expected_weights(p["position"], hidden_size))
+        return out
+
+    def state_floats(self) -> int:
+        return (self.taps - 1) * self.channels
+
+    def cache_spec(self):
+        kind = "window" if self.window is not None else "full"
+        if self.value_dim == self.head_dim:
+            return CacheSpec(kind, self.num_kv_heads, self.head_dim, self.window)
+        return SizedValueCacheSpec(kind, self.num_kv_heads, self.head_dim, self.window, self.value_dim)
+
+    def _paired(self, t: torch.Tensor) -> torch.Tensor:
+        """Rows of a q or k tensor (projection or convolution) with every head's rotary elements in paired order
+        (see ``PagedAttention._paired``: the rotation kernels take neighbours as pairs)."""
+        rot = self.position.rotary()
+        if rot is None or rot[1] == 0:
+            return t
+        rd, half, d = rot[1], rot[1] // 2, self.head_dim
+        order = torch.arange(d)
+        order[0:rd:2] = torch.arange(half)
+        order[1:rd:2] = torch.arange(half) + half
+        return t.view(t.shape[0] // d, d, -1)[:, order.to(t.device), :].reshape(t.shape)
+
+    def load_branch(self, get):
+        w = self.spec.weights
+        rows = [self._paired(get(w["q"])), self._paired(get(w["k"])), get(w["v"])]
+        if self.gate:
+            rows.append(get(w["gate"]))
+        conv = torch.cat([self._paired(get(w["q_conv"])), self._paired(get(w["k_conv"])), get(w["v_conv"])], dim=0)
+        self.conv_w = self._to_device(conv, torch.float32).t().contiguous()      # tap-major for the kernel
+        self.position.load_weights(get)
+        return torch.cat([self._to_device(t) for t in rows], dim=0).contiguous(), self._to_device(get(w["o"]))
+
+    def run(self, proj, col0, ctx, cache, out, out_col0, scale):
+        if not cache.writes:
+            raise ValueError("conv_attention: a call that reads another call's cache is not supported")
+        qkv = ops.causal_conv(proj, col0, self.channels, self.conv_w, None, cache.state, ctx.cu_seqlens, ctx.token_req,
+                              ctx.state_slots, ctx.num_requests, state_off=self.state_off, act=False)
+        rot = self.position.rotary()
+        inv_freq, rotary_dim, factor, table = None, 0, 1.0, None
+        if rot is not None:
+            inv_freq, rotary_dim, factor = rot
+            table = self.position.table(ctx) if hasattr(self.position, "table") else None
+        q = ops.rope_kv_write(qkv, ctx.positions, ctx.slot_mapping[cache.group], inv_freq, rotary_dim, factor, self.num_heads,
+                              self.num_kv_heads, self.head_dim, cache.k, cache.v, self.dtype, table, value_dim=self.value_dim)
+        a = ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
+                                ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len, ctx.num_single)
+        ops.sigmoid_gate(a, proj if self.gate else None, col0 + self.channels, scale, out, out_col0)
+
+
+register_part("mixer", "conv_attention", ConvAttention)

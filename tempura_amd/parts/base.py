@@ -122,6 +122,55 @@ class Mixer(Part):
         raise NotImplementedError
 
 
+class BranchMixer(Mixer):
+    """A mixer that lies between ONE input product and ONE output product: ``load_branch`` hands back the rows of
+    its input projection [rows, hidden] and its output projection [hidden, inner] (and keeps its small tensors
+    itself); ``run`` turns the float32 sums of the input product, found from column ``col0`` of ``proj`` on, into the
+    ``inner`` columns that enter the output product, times ``scale``, at column ``out_col0`` of ``out``.  Alone it
+    is an ordinary mixer; several of them side by side (the ``parallel`` mixer) share both products.  Its share of a
+    request's float32 state row starts at ``state_off`` (``state_floats()`` long)."""
+
+    graph_safe = True
+    returns_output = True      # with ``residual`` None the output comes back instead of being added
+    inner = 0
+    state_off = 0
+
+    def state_floats(self) -> int:
+        return 0
+
+    def load_branch(self, get):
+        raise NotImplementedError
+
+    def run(self, proj, col0, ctx, cache, out, out_col0, scale) -> None:
+        raise NotImplementedError
+
+    def state_spec(self):
+        n = self.state_floats()
+        return StateSpec((n,), torch.float32) if n else None
+
+    def load_weights(self, get):
+        from ..kernels import ops
+        w_in, w_out = self.load_branch(get)
+        self.w_in = ops.tile_weight(pad_rows(w_in, 16))
+        self.w_out = ops.tile_weight(w_out)
+
+    def forward(self, x, ctx, cache, residual=None):
+        from ..kernels import ops
+        proj = ops.linear(x, self.w_in, torch.float32)
+        act = torch.empty((proj.shape[0], self.inner), dtype=self.dtype, device=proj.device)
+        self.run(proj, 0, ctx, cache, act, 0, 1.0)
+        return ops.linear(act, self.w_out, torch.float32, residual=residual)
+
+
+def pad_rows(w: torch.Tensor, multiple: int) -> torch.Tensor:
+    """``w`` [rows, k] with zero rows added up to a multiple: the products then take the weight in their tiled
+    form; whoever reads the product's rows reads them by their stride and never sees the padding."""
+    pad = (-w.shape[0]) % multiple
+    if not pad:
+        return w.contiguous()
+    return torch.cat([w, torch.zeros((pad, w.shape[1]), dtype=w.dtype, device=w.device)], dim=0).contiguous()
+
+
 class FeedForward(Part):
     """Position-wise transform.  ``forward(x, ctx, residual)`` adds into ``residual``."""
 

@@ -212,3 +212,69 @@ class HyperBlock(ArrangedBlock):
 
 
 register_part("block", "hyper", HyperBlock)
+
+
+class SandwichBlock(ArrangedBlock):
+    """A norm before and a norm behind each sublayer: ``h += post(mixer(pre(h)))``, then, when the layer has a
+    feed-forward, ``h += post(ffn(pre(h)))``.  A constant that multiplies what enters the stream is the ``scale`` of
+    the norm behind the sublayer.  The norms behind the sublayers are RMS norms; one kernel norms a sublayer's
+    output, adds it into the stream and norms the stream for the next sublayer, also across layers (``entry_norm``
+    says what the block before needs for that)."""
+    ROLES = {"mixer_norm": "norm", "mixer": "mixer", "mixer_post_norm": "norm",
+             "ffn_norm": "norm", "ffn": "ffn", "ffn_post_norm": "norm"}
+    OPTIONAL = frozenset({"ffn_norm", "ffn", "ffn_post_norm"})
+    handoff = "sandwich"
+
+    def __init__(self, layer_spec, hidden_size, dtype, device):
+        super().__init__(layer_spec, hidden_size, dtype, device)
+        if len({self.ffn is None, self.ffn_norm is None, self.ffn_post_norm is None}) != 1:
+            raise ValueError("block 'sandwich': a feed-forward and its two norms come together")
+        for post in (self.mixer_post_norm, self.ffn_post_norm):
+            if post is not None and type(post).__name__ != "RMSNorm":
+                raise ValueError("block 'sandwich': the norm behind a sublayer must be an RMS norm")
+        self.hidden_size = hidden_size
+        self.dtype = dtype
+
+    @staticmethod
+    def _rms(norm):
+        """(weight, eps) of an RMS norm that the closing kernel can apply, else None."""
+        if type(norm).__name__ == "RMSNorm":
+            return norm.weight, norm.eps
+        return None
+
+    def entry_norm(self, m):
+        return self._rms(self.mixer_norm)
+
+    def _run(self, part, x, ctx, cache, n, device):
+        """A sublayer's output as a tensor of its own, float32 [tokens, hidden]."""
+        args = (x, ctx, cache) if cache is not None else (x, ctx)
+        if getattr(part, "returns_output", False):
+            return part.forward(*args, None)
+        y = torch.zeros((n, self.hidden_size), dtype=torch.float32, device=device)
+        part.forward(*args, y)
+        return y
+
+    def _close(self, h, y, post, opening):
+        """Norm ``y``, add it into the stream; with ``opening`` (weight, eps) also return the stream normed for the
+        next sublayer."""
+        if opening is None:
+            ops.norm_add(h, y, post.weight, post.eps)
+            return None
+        return ops.norm_add(h, y, post.weight, post.eps, opening[0], opening[1], self.dtype)
+
+    def forward(self, h, ctx, cache, x=None, next_norm=None):
+        n = h.shape[0]
+        if x is None:
+            x = self.mixer_norm.forward(h)
+        y = self._run(self.mixer, x, ctx, cache, n, h.device)
+        after = next_norm if isinstance(next_norm, tuple) else None
+        if self.ffn is None:
+            return self._close(h, y, self.mixer_post_norm, after)
+        x2 = self._close(h, y, self.mixer_post_norm, self._rms(self.ffn_norm))
+        if x2 is None:
+            x2 = self.ffn_norm.forward(h)
+        y2 = self._run(self.ffn, x2, ctx, None, n, h.device)
+        return self._close(h, y2, self.ffn_post_norm, after)
+
+
+register_part("block", "sandwich", SandwichBlock)

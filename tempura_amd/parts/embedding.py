@@ -9,13 +9,19 @@ output matrix the embedding matrix is used for it
 Two options beyond that: the embedding may add a sinusoidal position vector (``position: "sinusoid"`` with
 ``position_base`` b: element 2i of position p gets sin(p * b^(-2i / hidden)), element 2i + 1 the cosine), and the
 head may multiply its logits by a constant (``scale``).
+
+``bigram`` (``{"buckets", "mul_prev", "mul_cur"}``, tensor role ``bigram`` [buckets + 1, hidden]): a second row is
+added to every token's, chosen by a hash of the token before it and the token itself,
+(previous * mul_prev + token * mul_cur) mod buckets; a request's first token reads the last row.  The token before a
+step's first one is per-request state: the embedding says so with ``state_spec()`` (one int32 per request), the model
+asks for a state tensor on its behalf and hands it to ``forward``.
 """
 from __future__ import annotations
 
 import torch
 
 from ..kernels import ops
-from .base import Part, WeightInfo, register_part
+from .base import Part, StateSpec, WeightInfo, register_part
 
 
 class TokenEmbedding(Part):
@@ -34,16 +40,39 @@ class TokenEmbedding(Part):
             i = torch.arange((hidden_size + 1) // 2, dtype=torch.float64)
             # float64 on the host; the kernel forms the angle in float64 too
             self.inv_freq = torch.pow(torch.tensor(base, dtype=torch.float64), -2.0 * i / hidden_size).to(device)
+        self.bigram = spec.params.get("bigram")
+        self.bigram_table = None
+        if self.bigram is not None:
+            if kind is not None:
+                raise ValueError("embedding: a bigram table and a position vector together are not supported")
+            for key in ("buckets", "mul_prev", "mul_cur"):
+                if int(self.bigram[key]) < (1 if key == "buckets" else 0):
+                    raise ValueError(f"embedding: bigram {key} must be {'positive' if key == 'buckets' else 'non-negative'}")
 
     @classmethod
     def expected_weights(cls, spec, hidden_size, vocab_size):
-        return {spec.weights["weight"]: WeightInfo((vocab_size, hidden_size))}
+        out = {spec.weights["weight"]: WeightInfo((vocab_size, hidden_size))}
+        if spec.params.get("bigram") is not None:
+            out[spec.weights["bigram"]] = WeightInfo((int(spec.params["bigram"]["buckets"]) + 1, hidden_size))
+        return out
 
     def load_weights(self, get):
         self.weight = self._to_device(get(self.spec.weights["weight"]))
+        if self.bigram is not None:
+            self.bigram_table = self._to_device(get(self.spec.weights["bigram"]))
 
-    def forward(self, tokens, positions=None, streams: int = 1):
+    def state_spec(self):
+        """Per-request state of the embedding: the request's last token, for the bigram row of the next step's first."""
+        return StateSpec((1,), torch.int32) if self.bigram is not None else None
+
+    def forward(self, tokens, positions=None, streams: int = 1, ctx=None, state=None):
         """int32 [tokens] -> float32 [tokens, streams * hidden]: ``streams`` copies of the residual stream."""
+        if self.bigram is not None:
+            if streams != 1:
+                raise ValueError("embedding: a bigram table with several copies of the stream is not supported")
+            b = self.bigram
+            return ops.embed_bigram(tokens, self.weight, self.bigram_table, ctx.positions, ctx.token_req, ctx.cu_seqlens,
+                                    ctx.state_slots, state, ctx.num_requests, int(b["mul_prev"]), int(b["mul_cur"]), int(b["buckets"]))
         if self.inv_freq is None and streams == 1:
             return ops.embed(tokens, self.weight)
         return ops.embed(tokens, self.weight, positions, self.inv_freq, streams)

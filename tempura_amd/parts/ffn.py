@@ -105,5 +105,106 @@ class GatedFFN(FeedForward):
         return ops.linear(a, self.w2, torch.float32, residual=residual)
 
 
+class DenseMLP(FeedForward):
+    """``down(act(up(x)))`` without a gate; ``activation`` names the function (``gelu_tanh``, ``silu``), which reads
+    the float32 sums of the up product."""
+    graph_safe = True
+    returns_output = True      # with ``residual`` None the output comes back instead of being added
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        self.intermediate_size = int(spec.params["intermediate_size"])
+        self.activation = str(spec.params.get("activation", "gelu_tanh"))
+        if self.activation not in ops.ACTIVATIONS:
+            raise ValueError(f"mlp: activation {self.activation!r} unknown (known: {sorted(ops.ACTIVATIONS)})")
+        self.w_up = self.w_down = None
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        i, w = spec.params["intermediate_size"], spec.weights
+        return {w["up"]: WeightInfo((i, hidden_size)), w["down"]: WeightInfo((hidden_size, i))}
+
+    def load_weights(self, get):
+        w = self.spec.weights
+        self.w_up = ops.tile_weight(self._to_device(get(w["up"])))
+        self.w_down = ops.tile_weight(self._to_device(get(w["down"])))
+
+    def forward(self, x, ctx, residual=None):
+        u = ops.linear(x, self.w_up, torch.float32)
+        a = ops.activation(u, self.activation, self.dtype)
+        return ops.linear(a, self.w_down, torch.float32, residual=residual)
+
+
+class RoutedExperts(FeedForward):
+    """A mixture of ``experts`` gated feed-forwards (``down(silu(gate(x)) * up(x))``, no biases) of which every token
+    uses ``top``.  Router: logits = W_router x with float32 sums (in bfloat16 the operands are the bfloat16 rows and
+    the checkpoint's bfloat16 weights, whose products are exact in float32); scores s = softmax over all experts;
+    the choice adds ``correction`` to s and, with ``groups`` (``count`` equal groups of neighbouring experts,
+    ``keep``), only looks at the experts of the ``keep`` groups whose best choice score is largest; the weights are
+    the chosen experts' s, not renormalised.  The output is the weighted sum of the chosen experts' outputs.
+
+    Every expert runs over all rows of the step and a row's sum takes it with its weight, which is zero where the
+    expert was not chosen: a row's result does not depend on what else is in the batch, the experts are added in
+    ascending order, and nothing of the batch is read on the host (captured steps).  Tensor roles: ``router``,
+    ``correction``, and ``gate`` / ``up`` / ``down`` as name patterns with ``{}`` for the expert's number."""
+    graph_safe = True
+    returns_output = True
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        p = spec.params
+        self.experts = int(p["experts"])
+        self.top = int(p["top"])
+        self.intermediate_size = int(p["intermediate_size"])
+        g = p.get("groups")
+        self.groups = int(g["count"]) if g else 1
+        self.keep = int(g["keep"]) if g else 1
+        if not 0 < self.top <= self.experts:
+            raise ValueError("moe: top must lie between 1 and the number of experts")
+        if self.groups > 1 and (self.experts % self.groups != 0 or not 0 < self.keep <= self.groups
+                                or self.keep * (self.experts // self.groups) < self.top):
+            raise ValueError("moe: groups must divide the experts and the kept groups must hold at least top experts")
+        self.w_router = self.correction = None
+        self.w13, self.w2 = [], []
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        p, w = spec.params, spec.weights
+        i, e = p["intermediate_size"], p["experts"]
+        out = {w["router"]: WeightInfo((e, hidden_size)), w["correction"]: WeightInfo((e,))}
+        for n in range(e):
+            out[w["gate"].format(n)] = WeightInfo((i, hidden_size))
+            out[w["up"].format(n)] = WeightInfo((i, hidden_size))
+            out[w["down"].format(n)] = WeightInfo((hidden_size, i))
+        return out
+
+    def load_weights(self, get):
+        from .base import pad_rows
+        w = self.spec.weights
+        self.w_router = ops.tile_weight(pad_rows(self._to_device(get(w["router"])), 16))
+        self.correction = self._to_device(get(w["correction"]), torch.float32)
+        self.fused = self.dtype == torch.bfloat16 and ops.gated_layout_ok(self.intermediate_size, self.hidden_size)
+        self.w13, self.w2 = [], []
+        for n in range(self.experts):
+            gate, up = self._to_device(get(w["gate"].format(n))), self._to_device(get(w["up"].format(n)))
+            both = ops.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], dim=0).contiguous()
+            self.w13.append(ops.tile_weight(both))
+            self.w2.append(ops.tile_weight(self._to_device(get(w["down"].format(n)))))
+
+    def forward(self, x, ctx, residual=None):
+        logits = ops.linear(x, self.w_router, torch.float32)
+        dense, _, _ = ops.moe_route(logits, self.correction, self.experts, self.top, self.groups, self.keep)
+        y = residual      # (None: the first expert's share starts a new tensor)
+        for n in range(self.experts):
+            if self.fused:
+                a = ops.linear_swiglu(x, self.w13[n])
+            else:
+                a = ops.swiglu(ops.linear(x, self.w13[n], torch.float32), self.dtype)
+            y = ops.moe_accumulate(y, ops.linear(a, self.w2[n], torch.float32), dense, n)
+        return y if residual is None else None
+
+
+register_part("ffn", "mlp", DenseMLP)
+register_part("ffn", "moe", RoutedExperts)
 register_part("ffn", "swiglu", SwiGLU)
 register_part("ffn", "gated", GatedFFN)

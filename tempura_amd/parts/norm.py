@@ -2,6 +2,8 @@
 
 ``weight_offset`` (default 0) serves checkpoints that store the weight around zero: with 1.0 the stored tensor is
 the deviation from one.  The offset is added once, in float32, when the weight is loaded.
+``scale`` (default 1) multiplies the result: a norm behind a sublayer whose output enters the residual stream
+times a constant carries the constant here (the weight is multiplied once, when it is loaded).
 
 The reference multiplies ``x * scale * w`` with eps inside the square root,
 added to the mean (/root/reference/kernels/src/ggml/ops_llama.rs:201-216).
@@ -22,6 +24,7 @@ class RMSNorm(Norm):
         super().__init__(spec, hidden_size, dtype, device)
         self.eps = float(spec.params["eps"])
         self.weight_offset = float(spec.params.get("weight_offset", 0.0))
+        self.scale = float(spec.params.get("scale", 1.0))
         self.weight = None
 
     @classmethod
@@ -35,6 +38,8 @@ class RMSNorm(Norm):
         self.weight = self._to_device(get(self.spec.weights["weight"]), torch.float32)
         if self.weight_offset != 0.0:
             self.weight = (self.weight.double() + self.weight_offset).to(torch.float32)
+        if self.scale != 1.0:
+            self.weight = (self.weight.double() * self.scale).to(torch.float32)
 
     def forward(self, h, rows=None):
         return ops.rmsnorm(h, self.weight, self.eps, self.dtype, rows)

@@ -1,10 +1,14 @@
-"""Rotary position encoding with optional llama3 frequency scaling.
+"""Rotary position encoding with optional llama3 or YaRN frequency scaling.
 
 Pairs are split-half: element ``d`` rotates with element ``d + D/2`` by the angle
 ``pos * inv_freq[d]`` (/root/reference/kernels/src/rope.rs:18-53, 900-921), with
 ``inv_freq[d] = theta^(-2d/D)``.  The llama3 rule rescales each frequency by its
 wavelength (/root/reference/kernels/src/rope.rs:848-881).  The table is built in
-float64 on the host; kernels form the angle from the integer position in 64-bit
+float64 on the host.  The YaRN rule (``type: "yarn"`` with ``factor``, ``original``, ``fast``, ``slow``) blends
+each frequency f_i with f_i / factor by a ramp over the pair index: with
+c(t) = D ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(c(fast)), 0), hi = min(ceil(c(slow)), D - 1) and
+ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1) the frequency is f_i / factor * ramp_i + f_i (1 - ramp_i); what
+multiplies cosine and sine is the part's ``attn_factor``.  Kernels form the angle from the integer position in 64-bit
 and take sine and cosine of it, so no precision is lost at large positions.
 """
 from __future__ import annotations
@@ -28,6 +32,15 @@ def rotary_inv_freq(head_dim: int, theta: float, scaling=None, rotary_dim=None) 
     if scaling is None:
         return inv
     kind = scaling.get("rope_type", scaling.get("type"))
+    if kind == "yarn":
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def turn_index(turns: float) -> float:
+            return rd * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(theta)))
+        lo = max(math.floor(turn_index(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(turn_index(float(scaling["slow"]))), rd - 1)
+        ramp = torch.clamp((d - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return inv / factor * ramp + inv * (1.0 - ramp)
     if kind != "llama3":
         raise ValueError(f"rope scaling {kind!r} is not supported")
     factor = float(scaling["factor"])

@@ -74,21 +74,24 @@ class EmuOps:
                 v_cache[page, :, :, off] = k.to(v_cache.dtype)
         return q.reshape(n, num_heads, head_dim).to(q_dtype).contiguous()
 
-    def causal_conv(self, proj, col0, channels, weight, bias, state, cu_seqlens, token_req, state_slots, num_requests):
+    def causal_conv(self, proj, col0, channels, weight, bias, state, cu_seqlens, token_req, state_slots, num_requests,
+                    state_off=0, act=True):
         taps = weight.shape[0]                    # tap-major: [taps, channels]
         out = torch.zeros(proj.shape[0], channels, dtype=torch.float64)
         cu = cu_seqlens.tolist()
+        b = torch.zeros(channels, dtype=torch.float64) if bias is None else bias.double()
+        lo, hi = state_off, state_off + (taps - 1) * channels
         for r in range(num_requests):
-            a, b = cu[r], cu[r + 1]
-            if b <= a:
+            a, e = cu[r], cu[r + 1]
+            if e <= a:
                 continue
             slot = int(state_slots[r])
-            carried = state[slot, : (taps - 1) * channels].double().reshape(taps - 1, channels)
-            seq = torch.cat([carried, proj[a:b, col0: col0 + channels].double()], dim=0)
-            for t in range(b - a):
-                out[a + t] = (seq[t: t + taps] * weight.double()).sum(0) + bias.double()
-            state[slot, : (taps - 1) * channels] = seq[seq.shape[0] - (taps - 1):].reshape(-1).to(torch.float32)
-        return (out * torch.sigmoid(out)).to(torch.float32)
+            carried = state[slot, lo:hi].double().reshape(taps - 1, channels)
+            seq = torch.cat([carried, proj[a:e, col0: col0 + channels].double()], dim=0)
+            for t in range(e - a):
+                out[a + t] = (seq[t: t + taps] * weight.double()).sum(0) + b
+            state[slot, lo:hi] = seq[seq.shape[0] - (taps - 1):].reshape(-1).to(torch.float32)
+        return (out * torch.sigmoid(out) if act else out).to(torch.float32)
 
     def ssm_scan(self, xbc, proj, dt_col0, dt_bias, a_log, d_skip, state, state_off, cu_seqlens, state_slots, num_requests,
                  num_heads, head_dim, state_size, groups, max_run=None):
@@ -175,7 +178,7 @@ class EmuOps:
         return out
 
     def rope_kv_write(self, qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads, num_kv_heads,
-                      head_dim, k_cache, v_cache, q_dtype):
+                      head_dim, k_cache, v_cache, q_dtype, value_dim=None):
         n = qkv.shape[0]
         nrot = num_heads + (num_kv_heads if slots is not None else 0)
         x = qkv.double()[:, : nrot * head_dim].reshape(n, nrot, head_dim).clone()
@@ -191,7 +194,7 @@ class EmuOps:
         q = x[:, :num_heads].to(q_dtype).contiguous()
         if slots is not None:
             k = x[:, num_heads:]
-            v = qkv.double()[:, nrot * head_dim:].reshape(n, num_kv_heads, head_dim)
+            v = qkv.double()[:, nrot * head_dim:].reshape(n, num_kv_heads, value_dim or head_dim)
             ps = k_cache.shape[2]
             page, off = slots.long() // ps, slots.long() % ps
             k_cache[page, :, off] = k.to(k_cache.dtype)
@@ -203,7 +206,8 @@ class EmuOps:
         n, heads, d = q.shape
         kvh, ps = k_cache.shape[1], k_cache.shape[2]
         group = heads // kvh
-        out = torch.zeros(n, heads, d, dtype=torch.float64)
+        vd = v_cache.shape[2]
+        out = torch.zeros(n, heads, vd, dtype=torch.float64)
         cu = cu_seqlens.tolist()
         for r in range(block_tables.shape[0]):
             qs, qe = cu[r], cu[r + 1]
@@ -223,7 +227,119 @@ class EmuOps:
                         sc = sc + dist_bias[h].double()[dist]
                     p = torch.softmax(sc, dim=0)
                     out[t, h] = p @ V[lo: pos + 1, h // group]
-        return out.reshape(n, heads * d).to(q.dtype)
+        return out.reshape(n, heads * vd).to(q.dtype)
+
+    def embed_bigram(self, tokens, table, bigram, positions, token_req, cu_seqlens, state_slots, prev_state, num_requests,
+                     mul_prev, mul_cur, buckets):
+        out = torch.zeros(tokens.numel(), table.shape[1], dtype=torch.float64)
+        cu = cu_seqlens.tolist()
+        for r in range(num_requests):
+            slot = int(state_slots[r])
+            for t in range(cu[r], cu[r + 1]):
+                tok = int(tokens[t])
+                if int(positions[t]) == 0:
+                    row = buckets
+                else:
+                    prev = int(tokens[t - 1]) if t > cu[r] else int(prev_state[slot].reshape(-1)[0])
+                    row = (prev * mul_prev + tok * mul_cur) % buckets
+                out[t] = table[tok].double() + bigram[row].double()
+            if cu[r + 1] > cu[r]:
+                prev_state[slot] = int(tokens[cu[r + 1] - 1])
+        return out.to(torch.float32)
+
+    def sigmoid_gate(self, a, proj, gate_col0, scale, out, out_col0):
+        v = a.double()
+        if proj is not None:
+            v = v * torch.sigmoid(proj.double()[:, gate_col0: gate_col0 + a.shape[1]])
+        out[:, out_col0: out_col0 + a.shape[1]] = (v * scale).to(out.dtype)
+
+    def norm_add(self, h, y, weight, eps, next_weight=None, next_eps=0.0, out_dtype=None):
+        yd = y.double()
+        h.copy_((h.double() + yd / torch.sqrt((yd * yd).mean(-1, keepdim=True) + eps) * weight.double()).to(torch.float32))
+        if next_weight is None:
+            return None
+        return self.rmsnorm(h, next_weight, next_eps, out_dtype)
+
+    def activation(self, u, kind, out_dtype):
+        z = u.double()
+        if kind == "gelu_tanh":
+            v = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        else:
+            v = z * torch.sigmoid(z)
+        return v.to(out_dtype)
+
+    def moe_route(self, logits, correction, experts, top, groups, keep):
+        n = logits.shape[0]
+        s = torch.softmax(logits.double()[:, :experts], dim=-1)
+        dense = torch.zeros(n, experts, dtype=torch.float32)
+        ids = torch.zeros(n, top, dtype=torch.int32)
+        wts = torch.zeros(n, top, dtype=torch.float32)
+        for t in range(n):
+            ch = (s[t] + correction.double()).tolist()
+            if groups > 1:
+                per = experts // groups
+                score = [max(ch[g * per: (g + 1) * per]) for g in range(groups)]
+                kept = sorted(range(groups), key=lambda g: (-score[g], g))[:keep]
+                ch = [c if e // per in kept else float("-inf") for e, c in enumerate(ch)]
+            order = [e for e in sorted(range(experts), key=lambda e: (-ch[e], e)) if ch[e] != float("-inf")][:top]
+            for i, e in enumerate(order):
+                dense[t, e] = s[t, e]
+                ids[t, i] = e
+                wts[t, i] = s[t, e]
+        return dense, ids, wts
+
+    def moe_accumulate(self, y, part, dense, expert):
+        add = dense.double()[:, expert: expert + 1] * part.double()
+        if y is None:
+            return add.to(torch.float32)
+        y.copy_((y.double() + add).to(torch.float32))
+        return y
+
+    def lowrank_up(self, x, col0, weight_t, mode="plain", a_log=None, bias=None, per_head=0):
+        r = weight_t.shape[0]
+        v = x.double()[:, col0: col0 + r] @ weight_t.double()
+        if mode == "sigmoid":
+            v = torch.sigmoid(v)
+        elif mode == "decay":
+            rate = torch.exp(a_log.double()).repeat_interleave(per_head)
+            v = torch.exp(-rate * torch.nn.functional.softplus(v + bias.double()))
+        return v.to(torch.float32)
+
+    def delta_scan(self, qkv, decay, proj, beta_col0, state, state_off, cu_seqlens, state_slots, num_requests, heads, kv_heads,
+                   dim, vdim, q_scale, unit_eps):
+        n = qkv.shape[0]
+        rep = heads // kv_heads
+        x = qkv.double()
+        q = x[:, : kv_heads * dim].reshape(n, kv_heads, dim)
+        k = x[:, kv_heads * dim: 2 * kv_heads * dim].reshape(n, kv_heads, dim)
+        v = x[:, 2 * kv_heads * dim:].reshape(n, heads, vdim)
+        q = (q / torch.sqrt((q * q).sum(-1, keepdim=True) + unit_eps) * q_scale).repeat_interleave(rep, dim=1)
+        k = (k / torch.sqrt((k * k).sum(-1, keepdim=True) + unit_eps)).repeat_interleave(rep, dim=1)
+        beta = torch.sigmoid(proj.double()[:, beta_col0: beta_col0 + heads])
+        g = decay.double().reshape(n, heads, dim)
+        y = torch.zeros(n, heads, vdim, dtype=torch.float64)
+        cu = cu_seqlens.tolist()
+        size = heads * dim * vdim
+        for r in range(num_requests):
+            if cu[r + 1] <= cu[r]:
+                continue
+            slot = int(state_slots[r])
+            S = state[slot, state_off: state_off + size].double().reshape(heads, dim, vdim)
+            for t in range(cu[r], cu[r + 1]):
+                S = g[t][:, :, None] * S
+                u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
+                S = S + k[t][:, :, None] * u[:, None, :]
+                y[t] = torch.einsum("hdv,hd->hv", S, q[t])
+            state[slot, state_off: state_off + size] = S.reshape(-1).to(torch.float32)
+        return y.reshape(n, heads * vdim).to(torch.float32)
+
+    def head_norm_gate(self, o, weight, gate, eps, scale, heads, out, out_col0):
+        n, vdim = o.shape[0], o.shape[1] // heads
+        x = o.double().reshape(n, heads, vdim)
+        x = (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight.double()).reshape(n, heads * vdim)
+        if gate is not None:
+            x = x * gate.double()
+        out[:, out_col0: out_col0 + heads * vdim] = (x * scale).to(out.dtype)
 
     def swiglu(self, gu, out_dtype):
         i = gu.shape[1] // 2
