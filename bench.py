@@ -58,7 +58,7 @@ def parse_args():
     ap.add_argument("--mixed-chunk", type=int, default=512)
     ap.add_argument("--mixed-temperature", type=float, default=0.0, help="0: greedy; above: seeded sampling with top-k 50")
     ap.add_argument("--decode-target-blocks", type=int, default=None, help="tuning: blocks the split decode attention aims at")
-    ap.add_argument("--design", default=None, choices=["mifutar"],
+    ap.add_argument("--design", default=None, choices=["mifutar", "bomotar"],
                     help="instead of the headline: prefill and decode throughput of this design at layer sizes of real models, "
                          "beside Llama layers of equal size, with the time of every kernel entry point")
     ap.add_argument("--design-sizes", default="2048,4096", help="model widths of --design (comma separated)")
@@ -71,12 +71,16 @@ DESIGN_SIZES = {1024: (4096, 16, 64, 4), 2048: (8192, 32, 64, 8), 4096: (14336, 
 
 
 def design_bench(args) -> int:
-    """Prefill (one prompt, one step) and decode (a batch, captured steps) of the Mifutar design and of Llama layers
+    """Prefill (one prompt, one step) and decode (a batch, captured steps) of a design and of Llama layers
     of the same width, feed-forward width and attention heads, random weights, bfloat16 unless --dtype says
     otherwise.  A Mifutar model here has three state-space layers to one attention layer (window 1,024, four
-    streams); the Llama beside it has the same window.  Prints one JSON line."""
+    streams); the Llama beside it has the same window.  A Bomotar model here has, in every layer, an attention of the
+    Llama layer's heads (values as wide as keys, four taps, YaRN rotation) beside a delta rule of width / 128 heads
+    of 128 x 128 (low-rank projections of rank 64), and feed-forwards that alternate between a dense one and eight
+    experts of a quarter of its width, two a token out of two of four groups; it stands beside the Mifutar model and
+    the Llama layers (no window there).  Prints one JSON line."""
     import torch
-    from tempura_amd.config import LlamaConfig, MifutarConfig
+    from tempura_amd.config import BomotarConfig, LlamaConfig, MifutarConfig
     from tempura_amd.engine import Engine
     from tempura_amd.engine.loading import random_model
     from tempura_amd.engine.runner import StepEntry
@@ -84,6 +88,7 @@ def design_bench(args) -> int:
 
     rng = random.Random(0)
     window, vocab, T, batch = 1024, 32000, args.prompt_len, args.batch
+    design = args.design
     points = {}
 
     def say(msg):
@@ -99,8 +104,21 @@ def design_bench(args) -> int:
         return MifutarConfig.from_dict({"architecture": "Mifutar", "vocab": vocab, "width": width, "streams": 4, "logit_scale": 1.0,
                                         "norm": {"eps": 1e-6}, "layers": ls, "max_positions": 8192})
 
+    def bomotar_config(width, ff, heads, dim, kv, layers):
+        left = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "conv": 4, "scale": dim ** -0.5,
+                "rot": {"dims": dim, "base": 250000.0, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+        right = {"heads": width // 128, "kv_heads": width // 128, "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 64, "gate_rank": 64}
+        mixer = {"left": left, "right": right, "left_scale": 0.6, "right_scale": 0.9}
+        dense = {"kind": "dense", "ff": ff}
+        moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
+        ls = [{"type": "parallel", "mixer": mixer, "mlp": moe if i % 2 else dense} for i in range(layers)]
+        return BomotarConfig.from_dict({"architecture": "Bomotar", "vocab": vocab, "width": width, "residual_mult": 0.5,
+                                        "norm": {"eps": 1e-6}, "embedding": {"bigram": {"buckets": 65521, "mul_prev": 127, "mul_cur": 17}},
+                                        "layers": ls, "max_positions": 8192})
+
     def llama_config(width, ff, heads, dim, kv, layers):
-        return LlamaConfig(width, ff, layers, heads, kv, dim, vocab, 8192, 1e-5, 500000.0, None, False, sliding_window=window)
+        return LlamaConfig(width, ff, layers, heads, kv, dim, vocab, 8192, 1e-5, 500000.0, None, False,
+                           sliding_window=window if design == "mifutar" else None)
 
     def measure(model):
         pages = (batch + 1) * ((T + 600 + args.page_size - 1) // args.page_size) + 8
@@ -150,8 +168,11 @@ def design_bench(args) -> int:
             print(f"--design-sizes: no layer sizes for width {width} (known: {sorted(DESIGN_SIZES)})", file=sys.stderr)
             return 2
         ff, heads, dim, kv = DESIGN_SIZES[width]
-        for name, cfg in (("mifutar", mifutar_config(width, ff, heads, dim, kv, args.design_layers)),
-                          ("llama", llama_config(width, ff, heads, dim, kv, args.design_layers))):
+        models = [("mifutar", mifutar_config(width, ff, heads, dim, kv, args.design_layers)),
+                  ("llama", llama_config(width, ff, heads, dim, kv, args.design_layers))]
+        if design == "bomotar":
+            models.insert(0, ("bomotar", bomotar_config(width, ff, heads, dim, kv, args.design_layers)))
+        for name, cfg in models:
             say(f"{name} width {width}: building")
             model = random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
             points[f"{name}_w{width}"] = measure(model)
@@ -159,12 +180,14 @@ def design_bench(args) -> int:
                 f"decode {points[f'{name}_w{width}']['decode_tokens_per_s']} tok/s")
             del model
             torch.cuda.empty_cache()
-    first = f"mifutar_w{args.design_sizes.split(',')[0]}"
-    print(json.dumps({"metric": f"mifutar_prefill_tokens_per_s_T{T}", "value": points[first]["prefill_tokens_per_s"], "unit": "tokens/s",
+    first = f"{design}_w{args.design_sizes.split(',')[0]}"
+    print(json.dumps({"metric": f"{design}_prefill_tokens_per_s_T{T}", "value": points[first]["prefill_tokens_per_s"], "unit": "tokens/s",
                       "n_gpus": 1, "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
                       "data": "synthetic", "vs_baseline": None,
-                      "config": {"design": "Mifutar beside Llama layers of equal size", "layers": args.design_layers, "prompt": T,
-                                 "decode_batch": batch, "window": window}, "points": points}))
+                      "config": {"design": {"mifutar": "Mifutar beside Llama layers of equal size",
+                                            "bomotar": "Bomotar beside Mifutar and Llama layers of equal size"}[design],
+                                 "layers": args.design_layers, "prompt": T, "decode_batch": batch,
+                                 "window": window if design == "mifutar" else None}, "points": points}))
     return 0
 
 

@@ -26,16 +26,16 @@ __device__ inline float d_softplus(float v) { return fmaxf(v, 0.f) + log1pf(expf
 // qkv [n, row_stride] float32 holds, per token, q [kv_heads * dim] | k [kv_heads * dim] | v [heads * vdim] (after the
 // convolution and its activation); decay [n, heads * dim]; beta_raw is column beta_col0 + h of `proj`.
 //
-// A block owns one request, one head and CB = 256 / KS value columns; a thread holds PER consecutive key channels
-// of one column in registers, and the KS lanes of a wave that share a column (lane = ks * (64 / KS) + column) split
-// the key channels among them.  Tokens are taken TC at a time: their q, k, decay, v and beta are staged in LDS (rows
-// padded to KS * PER channels with q = k = 0, so the run itself needs no bounds), the unit norms and k . q are
-// formed there by a wave per token, then the run over the chunk is register arithmetic and 16-byte LDS reads that
-// most lanes share.
-#define DELTA_TC_MAX 16   // (fewer when the padded key size is large: the chunk has to fit 60 KB of LDS)
-
+// Two kernels.  delta_prep (a wave per token and key head, all tokens side by side) makes q and k unit vectors in
+// place and leaves k . q per token and key head.  delta_scan is the chain: a block owns one request, one head and
+// CB = 256 / KS value columns; a thread holds PER consecutive key channels of one column in registers, and the KS
+// neighbouring lanes that share a column split the key channels among them (their sums meet by row permutes, no
+// trip through LDS up to 16 lanes).  A wave has one instruction stream, so the time of a token is the number of
+// instructions a wave issues for it: few state entries a lane (8 up to a key size of 128) keep that near 60.
+// Tokens are taken TC at a time through LDS (rows padded to KS * PER channels with q = k = 0 and decay 1, so the
+// run itself needs no bounds); the next chunk's values travel from memory into registers while this chunk runs.
 struct DeltaArgs {
-  const float* qkv;
+  float* qkv;
   int row_stride;
   const float* decay;
   const float* proj;
@@ -45,30 +45,70 @@ struct DeltaArgs {
   const int* cu_seqlens;
   const int* state_slots;
   float* y;
+  float* kq;   // [n, kv_heads]
   int heads, kv_heads, dim, vdim;
-  int KS, TC;
   float q_scale, unit_eps;
 };
 
-template <int PER>
+__global__ __launch_bounds__(256) void delta_prep_kernel(DeltaArgs a, long pairs) {
+  const long p = (long)blockIdx.x * 4 + threadIdx.x / TP_WAVE;
+  const int lane = threadIdx.x % TP_WAVE;
+  if (p >= pairs) return;
+  const long t = p / a.kv_heads;
+  const int g = (int)(p % a.kv_heads);
+  float* q = a.qkv + (size_t)t * a.row_stride + (size_t)g * a.dim;
+  float* k = q + (size_t)a.kv_heads * a.dim;
+  float sq = 0.f, sk = 0.f;
+  for (int i = lane; i < a.dim; i += TP_WAVE) {
+    sq = fmaf(q[i], q[i], sq);
+    sk = fmaf(k[i], k[i], sk);
+  }
+  sq = wave_sum(sq);
+  sk = wave_sum(sk);
+  const float rq = a.q_scale / sqrtf(sq + a.unit_eps), rk = 1.0f / sqrtf(sk + a.unit_eps);
+  float dot = 0.f;
+  for (int i = lane; i < a.dim; i += TP_WAVE) {
+    const float qv = q[i] * rq, kv = k[i] * rk;
+    q[i] = qv;
+    k[i] = kv;
+    dot = fmaf(qv, kv, dot);
+  }
+  dot = wave_sum(dot);
+  if (lane == 0) a.kq[p] = dot;
+}
+
+// sum over KS neighbouring lanes (from a multiple of KS on); every lane gets it
+template <int KS>
+__device__ inline float column_sum(float v) {
+#define DPP_ADD(ctrl) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, false))
+  if (KS >= 2) DPP_ADD(0xB1);    // quad_perm [1, 0, 3, 2]
+  if (KS >= 4) DPP_ADD(0x4E);    // quad_perm [2, 3, 0, 1]
+  if (KS >= 8) DPP_ADD(0x141);   // row_half_mirror
+  if (KS >= 16) DPP_ADD(0x140);  // row_mirror
+#undef DPP_ADD
+  if (KS >= 32) v += __shfl_xor(v, 16, TP_WAVE);
+  return v;
+}
+
+template <int PER, int KS>
 __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaArgs a) {
-  extern __shared__ float lds[];
+  constexpr int DP = PER * KS, CW = TP_WAVE / KS, CB = 4 * CW;
+  constexpr int TC = DP <= 256 ? 16 : 4096 / DP;
+  constexpr int NI = (TC * DP + 255) / 256, NV = (TC * CB + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float qs[TC * DP];
+  __shared__ __attribute__((aligned(16))) float kk[TC * DP];
+  __shared__ __attribute__((aligned(16))) float gs[TC * DP];
+  __shared__ float vs[TC * CB];
+  __shared__ float bs[TC];
+  __shared__ float kqs[TC];
   const int r = blockIdx.x, h = blockIdx.y;
   const int start = a.cu_seqlens[r], len = a.cu_seqlens[r + 1] - start;
   if (len <= 0) return;
-  const int KS = a.KS, CW = TP_WAVE / KS, CB = 4 * CW, DP = KS * PER;
   const int tid = threadIdx.x, wave = tid / TP_WAVE, lane = tid % TP_WAVE;
-  const int ks = lane / CW, jl = wave * CW + lane % CW;
+  const int ks = lane % KS, jl = wave * CW + lane / KS;
   const int j = blockIdx.z * CB + jl;
   const bool col_ok = j < a.vdim;
   const int kvh = h / (a.heads / a.kv_heads);
-  const int TC = a.TC;
-  float* qs = lds;                         // [TC][DP]
-  float* kk = qs + TC * DP;          // [TC][DP]
-  float* gs = kk + TC * DP;          // [TC][DP]
-  float* vs = gs + TC * DP;          // [TC][CB]
-  float* bs = vs + TC * CB;          // [TC] beta
-  float* kq = bs + TC;               // [TC] k . q
 
   float* S_mem = a.state + (size_t)a.state_slots[r] * a.state_stride + a.state_off + (size_t)h * a.dim * a.vdim;
   float S[PER];
@@ -79,74 +119,91 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaArgs a) {
   }
   const int q_col = kvh * a.dim, k_col = (a.kv_heads + kvh) * a.dim, v_col = 2 * a.kv_heads * a.dim + h * a.vdim;
   const int out_width = a.heads * a.vdim;
+  const size_t decay_stride = (size_t)a.heads * a.dim;
 
+  float rq[NI], rk[NI], rg[NI], rv[NV], rb = 0.f, rkq = 0.f;
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      const int idx = it * 256 + tid;
+      const int t = idx / DP, i = idx % DP;
+      const bool in = idx < TC * DP && t0 + t < len && i < a.dim;
+      const size_t row = (size_t)(start + t0 + t);
+      rq[it] = in ? a.qkv[row * a.row_stride + q_col + i] : 0.f;
+      rk[it] = in ? a.qkv[row * a.row_stride + k_col + i] : 0.f;
+      rg[it] = in ? a.decay[row * decay_stride + (size_t)h * a.dim + i] : 1.f;
+    }
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int idx = it * 256 + tid;
+      const int t = idx / CB, c = idx % CB;
+      const int col = blockIdx.z * CB + c;
+      rv[it] = (idx < TC * CB && t0 + t < len && col < a.vdim) ? a.qkv[(size_t)(start + t0 + t) * a.row_stride + v_col + col] : 0.f;
+    }
+    if (tid < TC && t0 + tid < len) {
+      const size_t row = (size_t)(start + t0 + tid);
+      rb = d_sigmoid(a.proj[row * a.proj_stride + a.beta_col0 + h]);
+      rkq = a.kq[row * a.kv_heads + kvh];
+    }
+  };
+  fetch(0);
   for (int t0 = 0; t0 < len; t0 += TC) {
     const int tc = min(TC, len - t0);
     __syncthreads();   // the chunk before has been consumed
-    for (int idx = tid; idx < tc * DP; idx += 256) {
-      const int t = idx / DP, i = idx % DP;
-      const size_t row = (size_t)(start + t0 + t);
-      const bool in = i < a.dim;
-      qs[idx] = in ? a.qkv[row * a.row_stride + q_col + i] : 0.f;
-      kk[idx] = in ? a.qkv[row * a.row_stride + k_col + i] : 0.f;
-      gs[idx] = in ? a.decay[row * ((size_t)a.heads * a.dim) + (size_t)h * a.dim + i] : 1.f;
-    }
-    for (int idx = tid; idx < tc * CB; idx += 256) {
-      const int t = idx / CB, c = idx % CB;
-      const int col = blockIdx.z * CB + c;
-      vs[idx] = col < a.vdim ? a.qkv[(size_t)(start + t0 + t) * a.row_stride + v_col + col] : 0.f;
-    }
-    if (tid < tc) bs[tid] = d_sigmoid(a.proj[(size_t)(start + t0 + tid) * a.proj_stride + a.beta_col0 + h]);
-    __syncthreads();
-    // unit vectors and k . q: a wave per token
-    for (int t = wave; t < tc; t += 4) {
-      float sq = 0.f, sk = 0.f;
-      for (int i = lane; i < DP; i += TP_WAVE) {
-        const float qv = qs[t * DP + i], kv = kk[t * DP + i];
-        sq = fmaf(qv, qv, sq);
-        sk = fmaf(kv, kv, sk);
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      const int idx = it * 256 + tid;
+      if (idx < TC * DP) {
+        qs[idx] = rq[it];
+        kk[idx] = rk[it];
+        gs[idx] = rg[it];
       }
-      sq = wave_sum(sq);
-      sk = wave_sum(sk);
-      const float rq = a.q_scale / sqrtf(sq + a.unit_eps), rk = 1.0f / sqrtf(sk + a.unit_eps);
-      float dot = 0.f;
-      for (int i = lane; i < DP; i += TP_WAVE) {
-        const float qv = qs[t * DP + i] * rq, kv = kk[t * DP + i] * rk;
-        qs[t * DP + i] = qv;
-        kk[t * DP + i] = kv;
-        dot = fmaf(qv, kv, dot);
-      }
-      dot = wave_sum(dot);
-      if (lane == 0) kq[t] = dot;
+    }
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int idx = it * 256 + tid;
+      if (idx < TC * CB) vs[idx] = rv[it];
+    }
+    if (tid < TC) {
+      bs[tid] = rb;
+      kqs[tid] = rkq;
     }
     __syncthreads();
+    if (t0 + TC < len) fetch(t0 + TC);   // on its way while this chunk runs
     for (int t = 0; t < tc; ++t) {
       const float4* q4 = (const float4*)(qs + t * DP + ks * PER);
       const float4* k4 = (const float4*)(kk + t * DP + ks * PER);
       const float4* g4 = (const float4*)(gs + t * DP + ks * PER);
       float kr[PER];
-      float pred = 0.f, read = 0.f;
+      float pred[PER / 4], read[PER / 4];
 #pragma unroll
       for (int e4 = 0; e4 < PER / 4; ++e4) {
         const float4 q = q4[e4], k = k4[e4], g = g4[e4];
         const float qa[4] = {q.x, q.y, q.z, q.w}, ka[4] = {k.x, k.y, k.z, k.w}, ga[4] = {g.x, g.y, g.z, g.w};
+        float p = 0.f, rd = 0.f;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           const int e = e4 * 4 + c;
           kr[e] = ka[c];
           S[e] *= ga[c];
-          pred = fmaf(S[e], ka[c], pred);
-          read = fmaf(S[e], qa[c], read);
+          p = fmaf(S[e], ka[c], p);
+          rd = fmaf(S[e], qa[c], rd);
         }
+        pred[e4] = p;
+        read[e4] = rd;
       }
-      for (int o = CW; o < TP_WAVE; o <<= 1) {   // over the KS lanes of this column, the same order in every lane
-        pred += __shfl_xor(pred, o, TP_WAVE);
-        read += __shfl_xor(read, o, TP_WAVE);
+      float ps = pred[0], rs = read[0];
+#pragma unroll
+      for (int e4 = 1; e4 < PER / 4; ++e4) {   // (a fixed order: the same sums wherever the token stands)
+        ps += pred[e4];
+        rs += read[e4];
       }
-      const float u = bs[t] * (vs[t * CB + jl] - pred);
+      ps = column_sum<KS>(ps);
+      rs = column_sum<KS>(rs);
+      const float u = bs[t] * (vs[t * CB + jl] - ps);
 #pragma unroll
       for (int e = 0; e < PER; ++e) S[e] = fmaf(kr[e], u, S[e]);
-      if (ks == 0 && col_ok) a.y[(size_t)(start + t0 + t) * out_width + (size_t)h * a.vdim + j] = fmaf(u, kq[t], read);
+      if (ks == 0 && col_ok) a.y[(size_t)(start + t0 + t) * out_width + (size_t)h * a.vdim + j] = fmaf(u, kqs[t], rs);
     }
   }
 #pragma unroll
@@ -156,36 +213,43 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaArgs a) {
   }
 }
 
-extern "C" int tp_delta_scan(const float* qkv, int row_stride, const float* decay, const float* proj, int proj_stride,
+extern "C" int tp_delta_scan(float* qkv, int row_stride, const float* decay, const float* proj, int proj_stride,
                              int beta_col0, float* state, size_t state_stride, size_t state_off, const int* cu_seqlens,
-                             const int* state_slots, float* y, int n_req, int heads, int kv_heads, int dim, int vdim,
-                             float q_scale, float unit_eps, hipStream_t s) {
-  TP_REQUIRE(n_req >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0, "delta_scan: bad sizes");
+                             const int* state_slots, float* y, float* kq, int n, int n_req, int heads, int kv_heads, int dim,
+                             int vdim, float q_scale, float unit_eps, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && n_req >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0, "delta_scan: bad sizes");
   TP_REQUIRE(heads % kv_heads == 0, "delta_scan: %d heads is not a multiple of %d key heads", heads, kv_heads);
   TP_REQUIRE(dim <= 1024, "delta_scan: key size %d exceeds 1024", dim);
   TP_REQUIRE(row_stride >= 2 * kv_heads * dim + heads * vdim, "delta_scan: rows too short");
   TP_REQUIRE(state_stride >= state_off + (size_t)heads * dim * vdim, "delta_scan: state rows too short");
   TP_REQUIRE(heads <= 65535, "delta_scan: too many heads");
-  if (n_req == 0) return 0;
-  // PER key channels a lane, KS lanes a column (a power of two up to 32): the least padding of the key size
-  const int per = dim <= 64 ? 8 : (dim <= 256 ? 16 : 32);
+  if (n == 0 || n_req == 0) return 0;
+  DeltaArgs a{qkv, row_stride, decay, proj, proj_stride, beta_col0, state, state_stride, state_off, cu_seqlens, state_slots, y, kq,
+              heads, kv_heads, dim, vdim, q_scale, unit_eps};
+  const long pairs = (long)n * kv_heads;
+  TP_REQUIRE((pairs + 3) / 4 < 0x7fffffffL, "delta_scan: too many rows");
+  hipLaunchKernelGGL(delta_prep_kernel, dim3((unsigned)((pairs + 3) / 4)), dim3(256), 0, s, a, pairs);
+  // PER key channels a lane (8 up to a key size of 128, then 16, then 32), KS lanes a column (a power of two)
+  const int per = dim <= 128 ? 8 : (dim <= 256 ? 16 : 32);
   int ks = 1;
   while (ks * per < dim) ks *= 2;
-  TP_REQUIRE(ks <= 32, "delta_scan: key size %d does not fit", dim);
-  const int cb = 4 * (TP_WAVE / ks), dp = ks * per;
-  int tc = DELTA_TC_MAX;
-  while (tc > 1 && sizeof(float) * ((size_t)tc * (3 * dp + cb) + 2 * tc) > 60 * 1024) tc /= 2;
-  DeltaArgs a{qkv, row_stride, decay, proj, proj_stride, beta_col0, state, state_stride, state_off, cu_seqlens, state_slots, y,
-              heads, kv_heads, dim, vdim, ks, tc, q_scale, unit_eps};
+  const int cb = 4 * (TP_WAVE / ks);
   const dim3 grid(n_req, heads, (vdim + cb - 1) / cb);
   TP_REQUIRE(grid.z <= 65535, "delta_scan: too many value columns");
-  const size_t shmem = sizeof(float) * ((size_t)tc * (3 * dp + cb) + 2 * tc);
-  if (per == 8)
-    hipLaunchKernelGGL(delta_scan_kernel<8>, grid, dim3(256), shmem, s, a);
-  else if (per == 16)
-    hipLaunchKernelGGL(delta_scan_kernel<16>, grid, dim3(256), shmem, s, a);
-  else
-    hipLaunchKernelGGL(delta_scan_kernel<32>, grid, dim3(256), shmem, s, a);
+#define SCAN(P, K) hipLaunchKernelGGL((delta_scan_kernel<P, K>), grid, dim3(256), 0, s, a)
+  if (per == 8) {
+    if (ks == 1) SCAN(8, 1);
+    else if (ks == 2) SCAN(8, 2);
+    else if (ks == 4) SCAN(8, 4);
+    else if (ks == 8) SCAN(8, 8);
+    else SCAN(8, 16);
+  } else if (per == 16) {
+    SCAN(16, 16);
+  } else {
+    if (ks <= 16) SCAN(32, 16);
+    else SCAN(32, 32);
+  }
+#undef SCAN
   TP_CHECK_LAUNCH("delta_scan");
   return 0;
 }
@@ -201,21 +265,30 @@ __global__ __launch_bounds__(256) void lowrank_up_kernel(const float* __restrict
                                                          const float* __restrict__ wt, float* __restrict__ out, int n,
                                                          int n_out, int mode, const float* __restrict__ a_log,
                                                          const float* __restrict__ bias, int per_head) {
-  extern __shared__ float xs[];   // [LR_ROWS][rank]
+  extern __shared__ __attribute__((aligned(16))) float xs[];   // [LR_ROWS][rank4]: rows padded with zeros to four
+  const int rank4 = (rank + 3) & ~3;
   const int t0 = blockIdx.x * LR_ROWS, c = blockIdx.y * 256 + threadIdx.x;
-  for (int idx = threadIdx.x; idx < LR_ROWS * rank; idx += 256) {
-    const int t = idx / rank, i = idx % rank;
-    xs[idx] = t0 + t < n ? x[(size_t)(t0 + t) * x_stride + col0 + i] : 0.f;
+  for (int idx = threadIdx.x; idx < LR_ROWS * rank4; idx += 256) {
+    const int t = idx / rank4, i = idx % rank4;
+    xs[idx] = (t0 + t < n && i < rank) ? x[(size_t)(t0 + t) * x_stride + col0 + i] : 0.f;
   }
   __syncthreads();
   if (c >= n_out) return;
   float acc[LR_ROWS];
 #pragma unroll
   for (int t = 0; t < LR_ROWS; ++t) acc[t] = 0.f;
-  for (int i = 0; i < rank; ++i) {
-    const float w = wt[(size_t)i * n_out + c];
+  for (int i = 0; i < rank4; i += 4) {   // (ascending i for every row: the same sums wherever the row stands)
+    float w[4];
 #pragma unroll
-    for (int t = 0; t < LR_ROWS; ++t) acc[t] = fmaf(xs[t * rank + i], w, acc[t]);
+    for (int d = 0; d < 4; ++d) w[d] = i + d < rank ? wt[(size_t)(i + d) * n_out + c] : 0.f;
+#pragma unroll
+    for (int t = 0; t < LR_ROWS; ++t) {
+      const float4 v = *(const float4*)(xs + t * rank4 + i);
+      acc[t] = fmaf(v.x, w[0], acc[t]);
+      acc[t] = fmaf(v.y, w[1], acc[t]);
+      acc[t] = fmaf(v.z, w[2], acc[t]);
+      acc[t] = fmaf(v.w, w[3], acc[t]);
+    }
   }
   float rate = 0.f, b = 0.f;
   if (mode == 2) {
@@ -241,7 +314,7 @@ extern "C" int tp_lowrank_up(const float* x, int x_stride, int col0, int rank, c
   if (n == 0) return 0;
   const dim3 grid((n + LR_ROWS - 1) / LR_ROWS, (n_out + 255) / 256);
   TP_REQUIRE(grid.y <= 65535, "lowrank_up: too many columns");
-  hipLaunchKernelGGL(lowrank_up_kernel, grid, dim3(256), sizeof(float) * LR_ROWS * rank, s, x, x_stride, col0, rank, wt, out, n,
+  hipLaunchKernelGGL(lowrank_up_kernel, grid, dim3(256), sizeof(float) * LR_ROWS * ((rank + 3) & ~3), s, x, x_stride, col0, rank, wt, out, n,
                      n_out, mode, a_log, bias, per_head);
   TP_CHECK_LAUNCH("lowrank_up");
   return 0;

@@ -75,21 +75,59 @@ __global__ void sigmoid_gate_kernel(const T* __restrict__ a, const float* __rest
   from_float(out + t * out_stride + out_col0 + c, v * scale);
 }
 
+// the same, four neighbouring columns a thread (every width, stride and first column a multiple of four)
+template <typename T>
+__global__ void sigmoid_gate4_kernel(const T* __restrict__ a, const float* __restrict__ proj, int proj_stride, int gate_col0,
+                                     float scale, T* __restrict__ out, int out_stride, int out_col0, int width, size_t total4) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total4) return;
+  const int w4 = width / 4;
+  const size_t t = i / w4;
+  const int c = (int)(i % w4) * 4;
+  float v[4];
+  if constexpr (sizeof(T) == 2) {
+    const uint2 raw = *(const uint2*)(a + t * width + c);
+    bf16_t h0{(uint16_t)(raw.x & 0xffff)}, h1{(uint16_t)(raw.x >> 16)}, h2{(uint16_t)(raw.y & 0xffff)}, h3{(uint16_t)(raw.y >> 16)};
+    v[0] = bf16_to_float(h0); v[1] = bf16_to_float(h1); v[2] = bf16_to_float(h2); v[3] = bf16_to_float(h3);
+  } else {
+    const float4 raw = *(const float4*)(a + t * width + c);
+    v[0] = raw.x; v[1] = raw.y; v[2] = raw.z; v[3] = raw.w;
+  }
+  if (proj != nullptr) {
+    const float4 g = *(const float4*)(proj + t * proj_stride + gate_col0 + c);
+    v[0] *= l_sigmoid(g.x); v[1] *= l_sigmoid(g.y); v[2] *= l_sigmoid(g.z); v[3] *= l_sigmoid(g.w);
+  }
+  from_float4(out + t * out_stride + out_col0 + c, v[0] * scale, v[1] * scale, v[2] * scale, v[3] * scale);
+}
+
 extern "C" int tp_sigmoid_gate(const void* a, int dt, const float* proj, int proj_stride, int gate_col0, float scale, void* out,
                                int out_stride, int out_col0, int n, int width, hipStream_t s) {
   TP_REQUIRE(n >= 0 && width > 0 && out_col0 >= 0 && out_stride >= out_col0 + width, "sigmoid_gate: bad sizes");
   TP_REQUIRE(proj == nullptr || (gate_col0 >= 0 && proj_stride >= gate_col0 + width), "sigmoid_gate: gate rows too short");
+  TP_REQUIRE(dt == TP_F32 || dt == TP_BF16, "sigmoid_gate: unknown dtype %d", dt);
   if (n == 0) return 0;
-  const size_t total = (size_t)n * width;
-  const dim3 grid((unsigned)((total + 255) / 256));
-  if (dt == TP_F32)
-    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, grid, dim3(256), 0, s, (const float*)a, proj, proj_stride, gate_col0, scale,
-                       (float*)out, out_stride, out_col0, width, total);
-  else if (dt == TP_BF16)
-    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)a, proj, proj_stride, gate_col0, scale,
-                       (bf16_t*)out, out_stride, out_col0, width, total);
-  else
-    TP_REQUIRE(false, "sigmoid_gate: unknown dtype %d", dt);
+  const size_t esz = dt == TP_F32 ? 4 : 2;
+  const bool four = width % 4 == 0 && out_stride % 4 == 0 && out_col0 % 4 == 0 && (proj == nullptr || (proj_stride % 4 == 0 && gate_col0 % 4 == 0)) &&
+                    (uintptr_t)a % 16 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)proj % 16 == 0 && esz * 4 <= 16;
+  if (four) {
+    const size_t total4 = (size_t)n * (width / 4);
+    const dim3 grid((unsigned)((total4 + 255) / 256));
+    if (dt == TP_F32)
+      hipLaunchKernelGGL(sigmoid_gate4_kernel<float>, grid, dim3(256), 0, s, (const float*)a, proj, proj_stride, gate_col0, scale,
+                         (float*)out, out_stride, out_col0, width, total4);
+    else
+      hipLaunchKernelGGL(sigmoid_gate4_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)a, proj, proj_stride, gate_col0, scale,
+                         (bf16_t*)out, out_stride, out_col0, width, total4);
+  } else {
+    const size_t total = (size_t)n * width;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (dt == TP_F32)
+      hipLaunchKernelGGL(sigmoid_gate_kernel<float>, grid, dim3(256), 0, s, (const float*)a, proj, proj_stride, gate_col0, scale,
+                         (float*)out, out_stride, out_col0, width, total);
+    else
+      hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)a, proj, proj_stride, gate_col0, scale,
+                         (bf16_t*)out, out_stride, out_col0, width, total);
+  }
   TP_CHECK_LAUNCH("sigmoid_gate");
   return 0;
 }
@@ -139,22 +177,40 @@ extern "C" int tp_norm_add(float* h, const float* y, const float* w, float eps, 
 
 // ---- a plain activation -----------------------------------------------------------------------
 // kind 0: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))); kind 1: SiLU.
+__device__ inline float act_f(float z, int kind) {
+  if (kind == 0) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return z * l_sigmoid(z);
+}
+
 template <typename TI, typename TO>
 __global__ void activation_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t total, int kind) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total) return;
-  const float z = to_float(in[i]);
-  float v;
-  if (kind == 0)
-    v = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-  else
-    v = z * l_sigmoid(z);
-  from_float(out + i, v);
+  from_float(out + i, act_f(to_float(in[i]), kind));
+}
+
+// float32 in, four neighbouring elements a thread
+template <typename TO>
+__global__ void activation4_kernel(const float* __restrict__ in, TO* __restrict__ out, size_t total4, int kind) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total4) return;
+  const float4 z = *(const float4*)(in + 4 * i);
+  from_float4(out + 4 * i, act_f(z.x, kind), act_f(z.y, kind), act_f(z.z, kind), act_f(z.w, kind));
 }
 
 extern "C" int tp_activation(const void* in, int in_dt, void* out, int out_dt, size_t total, int kind, hipStream_t s) {
   TP_REQUIRE(kind == 0 || kind == 1, "activation: unknown kind %d", kind);
   if (total == 0) return 0;
+  if (in_dt == TP_F32 && total % 4 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0 && (out_dt == TP_F32 || out_dt == TP_BF16)) {
+    const size_t total4 = total / 4;
+    const dim3 grid4((unsigned)((total4 + 255) / 256));
+    if (out_dt == TP_F32)
+      hipLaunchKernelGGL(activation4_kernel<float>, grid4, dim3(256), 0, s, (const float*)in, (float*)out, total4, kind);
+    else
+      hipLaunchKernelGGL(activation4_kernel<bf16_t>, grid4, dim3(256), 0, s, (const float*)in, (bf16_t*)out, total4, kind);
+    TP_CHECK_LAUNCH("activation");
+    return 0;
+  }
   const dim3 grid((unsigned)((total + 255) / 256));
 #define ACT(TI, TO) hipLaunchKernelGGL((activation_kernel<TI, TO>), grid, dim3(256), 0, s, (const TI*)in, (TO*)out, total, kind)
   if (in_dt == TP_F32 && out_dt == TP_F32)
@@ -322,5 +378,96 @@ extern "C" int tp_moe_accumulate(float* y, const float* part, const float* dense
   hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, y, part, dense, experts, e,
                      width, total, first);
   TP_CHECK_LAUNCH("moe_accumulate");
+  return 0;
+}
+
+// ---- rows sorted by expert --------------------------------------------------------------------
+// For steps of many rows the chosen (token, expert) pairs are brought into the order of the experts, so that
+// every expert is one product over its own rows.  ids [n, top] lists each token's experts; pair p = t * top + k.
+// moe_plan: counts[e] = pairs of expert e, rank[p] = how many pairs of the same expert come before p (in the order
+// of p), so the order inside an expert's rows is the order of the tokens whatever else the batch holds; then
+// offsets[e] = pairs of the experts before e.  One block per expert walks all pairs; a one-block kernel adds up.
+__global__ __launch_bounds__(256) void moe_rank_kernel(const int* __restrict__ ids, int pairs, int* __restrict__ counts,
+                                                       int* __restrict__ rank) {
+  __shared__ int wave_total[4];
+  const int e = blockIdx.x, lane = threadIdx.x % TP_WAVE, wave = threadIdx.x / TP_WAVE;
+  int base = 0;
+  for (int p0 = 0; p0 < pairs; p0 += 256) {
+    const int p = p0 + threadIdx.x;
+    const bool mine = p < pairs && ids[p] == e;
+    const unsigned long long mask = __ballot(mine);
+    const int before = __popcll(mask & ((1ull << lane) - 1ull));
+    __syncthreads();   // (the totals of the chunk before have been read)
+    if (lane == 0) wave_total[wave] = __popcll(mask);
+    __syncthreads();
+    int prior = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      if (w < wave) prior += wave_total[w];
+      total += wave_total[w];
+    }
+    if (mine) rank[p] = base + prior + before;
+    base += total;
+  }
+  if (threadIdx.x == 0) counts[e] = base;
+}
+
+__global__ void moe_offsets_kernel(const int* __restrict__ counts, int* __restrict__ offsets, int experts) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int acc = 0;
+  for (int e = 0; e < experts; ++e) {
+    offsets[e] = acc;
+    acc += counts[e];
+  }
+  offsets[experts] = acc;
+}
+
+extern "C" int tp_moe_plan(const int* ids, int n, int top, int experts, int* counts, int* offsets, int* rank, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && top > 0 && experts > 0 && (long)n * top < 0x7fffffffL, "moe_plan: bad sizes");
+  hipLaunchKernelGGL(moe_rank_kernel, dim3(experts), dim3(256), 0, s, ids, n * top, counts, rank);
+  hipLaunchKernelGGL(moe_offsets_kernel, dim3(1), dim3(64), 0, s, counts, offsets, experts);
+  TP_CHECK_LAUNCH("moe_plan");
+  return 0;
+}
+
+// xg[offsets[ids[p]] + rank[p]] = x[p / top] (rows of 4-byte words); row_of[p] remembers the place.
+__global__ void moe_gather_kernel(const uint32_t* __restrict__ x, const int* __restrict__ ids, const int* __restrict__ rank,
+                                  const int* __restrict__ offsets, uint32_t* __restrict__ xg, int* __restrict__ row_of, int top,
+                                  int words) {
+  const int p = blockIdx.x;
+  const int row = offsets[ids[p]] + rank[p];
+  if (threadIdx.x == 0) row_of[p] = row;
+  const uint32_t* src = x + (size_t)(p / top) * words;
+  uint32_t* dst = xg + (size_t)row * words;
+  for (int c = threadIdx.x; c < words; c += blockDim.x) dst[c] = src[c];
+}
+
+extern "C" int tp_moe_gather(const void* x, const int* ids, const int* rank, const int* offsets, void* xg, int* row_of, int n, int top,
+                             int row_bytes, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && top > 0 && row_bytes > 0 && row_bytes % 4 == 0, "moe_gather: rows must be a multiple of four bytes");
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(moe_gather_kernel, dim3(n * top), dim3(row_bytes / 4 >= 256 ? 256 : 64), 0, s, (const uint32_t*)x, ids, rank, offsets,
+                     (uint32_t*)xg, row_of, top, row_bytes / 4);
+  TP_CHECK_LAUNCH("moe_gather");
+  return 0;
+}
+
+// y[t] (+)= sum_k weights[t, k] * yg[row_of[t, k]], k ascending.
+__global__ void moe_scatter_kernel(const float* __restrict__ yg, const int* __restrict__ row_of, const float* __restrict__ weights,
+                                   float* __restrict__ y, int top, int width, int accumulate) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float acc = accumulate ? y[(size_t)t * width + c] : 0.f;
+    for (int k = 0; k < top; ++k) acc = fmaf(weights[(size_t)t * top + k], yg[(size_t)row_of[(size_t)t * top + k] * width + c], acc);
+    y[(size_t)t * width + c] = acc;
+  }
+}
+
+extern "C" int tp_moe_scatter(const float* yg, const int* row_of, const float* weights, float* y, int n, int top, int width,
+                              int accumulate, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && top > 0 && width > 0, "moe_scatter: bad sizes");
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(moe_scatter_kernel, dim3(n), dim3(width >= 256 ? 256 : 64), 0, s, yg, row_of, weights, y, top, width, accumulate);
+  TP_CHECK_LAUNCH("moe_scatter");
   return 0;
 }

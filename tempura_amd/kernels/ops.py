@@ -1325,7 +1325,8 @@ def delta_scan(qkv: torch.Tensor, decay: torch.Tensor, proj: torch.Tensor, beta_
     [kv_heads * dim] and v [heads * vdim]; q and k are made unit vectors per head (x / sqrt(sum x^2 + unit_eps), q times
     ``q_scale``); beta = sigmoid(proj[:, beta_col0 + h]); ``decay`` float32 [n, heads * dim].  Per head, with S
     [dim, vdim] at ``state[slot, state_off:]``:  S <- decay * S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
-    Returns o float32 [n, heads * vdim]; the state is left as the run leaves it."""
+    Returns o float32 [n, heads * vdim]; the state is left as the run leaves it.  (q and k of ``qkv`` are left as
+    unit vectors: the rows are a temporary of the caller's.)"""
     if _backend is not None:
         return _backend.delta_scan(qkv, decay, proj, beta_col0, state, state_off, cu_seqlens, state_slots, num_requests, heads,
                                    kv_heads, dim, vdim, q_scale, unit_eps)
@@ -1340,9 +1341,10 @@ def delta_scan(qkv: torch.Tensor, decay: torch.Tensor, proj: torch.Tensor, beta_
     _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
     _i32(state_slots, num_requests, "state_slots")
     y = torch.empty((n, heads * vdim), dtype=torch.float32, device=qkv.device)
+    kq = torch.empty((n, kv_heads), dtype=torch.float32, device=qkv.device)      # k . q per token and key head
     _call("tp_delta_scan", _ptr(qkv), qkv.shape[1], _ptr(decay), _ptr(proj), proj.shape[1], int(beta_col0), _ptr(state),
-          ctypes.c_size_t(state.shape[1]), ctypes.c_size_t(state_off), _ptr(cu_seqlens), _ptr(state_slots), _ptr(y), int(num_requests),
-          int(heads), int(kv_heads), int(dim), int(vdim), ctypes.c_float(q_scale), ctypes.c_float(unit_eps), _stream())
+          ctypes.c_size_t(state.shape[1]), ctypes.c_size_t(state_off), _ptr(cu_seqlens), _ptr(state_slots), _ptr(y), _ptr(kq), n,
+          int(num_requests), int(heads), int(kv_heads), int(dim), int(vdim), ctypes.c_float(q_scale), ctypes.c_float(unit_eps), _stream())
     return y
 
 
@@ -1360,3 +1362,48 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.T
     _need(out.dim() == 2 and out.shape[0] == n and 0 <= out_col0 and out_col0 + o.shape[1] <= out.shape[1], "head_norm_gate: output rows too short")
     _call("tp_head_norm_gate", _ptr(o), _ptr(weight), _ptr(gate), ctypes.c_float(eps), ctypes.c_float(scale), _ptr(out), _dt(out),
           out.shape[1], int(out_col0), n, int(heads), vdim, _stream())
+
+
+def moe_plan(ids: torch.Tensor, experts: int):
+    """Where every chosen (token, expert) pair goes when the pairs are brought into the order of the experts:
+    ``ids`` int32 [n, top] -> (counts int32 [experts], offsets int32 [experts + 1], rank int32 [n, top]); pair (t, k)
+    goes to row offsets[ids[t, k]] + rank[t, k], the pairs of one expert keeping the order of the tokens."""
+    if _backend is not None:
+        return _backend.moe_plan(ids, experts)
+    _dev_ok(ids)
+    _need(ids.dtype == torch.int32 and ids.dim() == 2, "moe_plan: ids must be int32 [n, top]")
+    counts = torch.empty((experts,), dtype=torch.int32, device=ids.device)
+    offsets = torch.empty((experts + 1,), dtype=torch.int32, device=ids.device)
+    rank = torch.empty(ids.shape, dtype=torch.int32, device=ids.device)
+    _call("tp_moe_plan", _ptr(ids), ids.shape[0], ids.shape[1], int(experts), _ptr(counts), _ptr(offsets), _ptr(rank), _stream())
+    return counts, offsets, rank
+
+
+def moe_gather(x: torch.Tensor, ids: torch.Tensor, rank: torch.Tensor, offsets: torch.Tensor):
+    """(rows [n * top, width] of ``x`` [n, width] in the order of the experts, row_of int32 [n, top]: the row of pair (t, k))."""
+    if _backend is not None:
+        return _backend.moe_gather(x, ids, rank, offsets)
+    _dev_ok(x, ids, rank, offsets)
+    n, top = ids.shape
+    _need(x.dim() == 2 and x.shape[0] == n and (x.shape[1] * x.element_size()) % 4 == 0, "moe_gather: rows must be a multiple of four bytes")
+    _need(rank.dtype == torch.int32 and tuple(rank.shape) == (n, top) and offsets.dtype == torch.int32, "moe_gather: bad plan")
+    xg = torch.empty((n * top, x.shape[1]), dtype=x.dtype, device=x.device)
+    row_of = torch.empty((n, top), dtype=torch.int32, device=x.device)
+    _call("tp_moe_gather", _ptr(x), _ptr(ids), _ptr(rank), _ptr(offsets), _ptr(xg), _ptr(row_of), n, top, x.shape[1] * x.element_size(), _stream())
+    return xg, row_of
+
+
+def moe_scatter(yg: torch.Tensor, row_of: torch.Tensor, weights: torch.Tensor, y: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y[t] (+)= sum_k weights[t, k] * yg[row_of[t, k]] (k ascending); ``y`` None: a new tensor."""
+    if _backend is not None:
+        return _backend.moe_scatter(yg, row_of, weights, y)
+    _dev_ok(yg, row_of, weights, y)
+    n, top = row_of.shape
+    _need(yg.dtype == torch.float32 and yg.dim() == 2 and yg.shape[0] == n * top and weights.dtype == torch.float32
+          and tuple(weights.shape) == (n, top) and row_of.dtype == torch.int32, "moe_scatter: bad operands")
+    acc = y is not None
+    if not acc:
+        y = torch.empty((n, yg.shape[1]), dtype=torch.float32, device=yg.device)
+    _need(y.dtype == torch.float32 and tuple(y.shape) == (n, yg.shape[1]), "moe_scatter: y must be float32 [n, width]")
+    _call("tp_moe_scatter", _ptr(yg), _ptr(row_of), _ptr(weights), _ptr(y), n, top, yg.shape[1], int(acc), _stream())
+    return y

@@ -143,9 +143,13 @@ class RoutedExperts(FeedForward):
     ``keep``), only looks at the experts of the ``keep`` groups whose best choice score is largest; the weights are
     the chosen experts' s, not renormalised.  The output is the weighted sum of the chosen experts' outputs.
 
-    Every expert runs over all rows of the step and a row's sum takes it with its weight, which is zero where the
-    expert was not chosen: a row's result does not depend on what else is in the batch, the experts are added in
-    ascending order, and nothing of the batch is read on the host (captured steps).  Tensor roles: ``router``,
+    Two ways through the experts.  A step of single tokens (decoding; it may be captured): every expert runs over
+    all rows and a row's sum takes it with its weight, which is zero where the expert was not chosen; the experts
+    are added in ascending order and nothing of the batch is read on the host.  A step with portions of prompts: the
+    chosen (token, expert) pairs are brought into the order of the experts, the host reads how many rows each expert
+    has (the one wait of the layer), every expert with rows is one pair of products over its rows, and a token's
+    sum adds its experts' rows in the order of its choice.  Either way a row's result does not depend on what else
+    is in the batch; the two ways differ in rounding only.  Tensor roles: ``router``,
     ``correction``, and ``gate`` / ``up`` / ``down`` as name patterns with ``{}`` for the expert's number."""
     graph_safe = True
     returns_output = True
@@ -191,16 +195,28 @@ class RoutedExperts(FeedForward):
             self.w13.append(ops.tile_weight(both))
             self.w2.append(ops.tile_weight(self._to_device(get(w["down"].format(n)))))
 
+    def _expert(self, n, rows):
+        if self.fused:
+            return ops.linear_swiglu(rows, self.w13[n])
+        return ops.swiglu(ops.linear(rows, self.w13[n], torch.float32), self.dtype)
+
     def forward(self, x, ctx, residual=None):
         logits = ops.linear(x, self.w_router, torch.float32)
-        dense, _, _ = ops.moe_route(logits, self.correction, self.experts, self.top, self.groups, self.keep)
-        y = residual      # (None: the first expert's share starts a new tensor)
-        for n in range(self.experts):
-            if self.fused:
-                a = ops.linear_swiglu(x, self.w13[n])
-            else:
-                a = ops.swiglu(ops.linear(x, self.w13[n], torch.float32), self.dtype)
-            y = ops.moe_accumulate(y, ops.linear(a, self.w2[n], torch.float32), dense, n)
+        dense, ids, weights = ops.moe_route(logits, self.correction, self.experts, self.top, self.groups, self.keep)
+        if getattr(ctx, "max_q_len", 1) <= 1:
+            y = residual      # (None: the first expert's share starts a new tensor)
+            for n in range(self.experts):
+                y = ops.moe_accumulate(y, ops.linear(self._expert(n, x), self.w2[n], torch.float32), dense, n)
+            return y if residual is None else None
+        counts, offsets, rank = ops.moe_plan(ids, self.experts)
+        xg, row_of = ops.moe_gather(x, ids, rank, offsets)
+        yg = torch.zeros((xg.shape[0], self.hidden_size), dtype=torch.float32, device=xg.device)
+        at = 0
+        for n, m in enumerate(counts.tolist()):      # (the host waits here for the router)
+            if m:
+                ops.linear(self._expert(n, xg[at: at + m]), self.w2[n], torch.float32, residual=yg[at: at + m])
+                at += m
+        y = ops.moe_scatter(yg, row_of, weights, residual)
         return y if residual is None else None
 
 

@@ -83,10 +83,12 @@ def config_json(name: str) -> dict:
     return cfg
 
 
-def make_weights(name: str, seed: int = 0, sharp: float = 1.0) -> Dict[str, torch.Tensor]:
+def make_weights(name: str, seed: int = 0, sharp: float = 1.0, apart: bool = False) -> Dict[str, torch.Tensor]:
     """bfloat16 tensors by checkpoint name, drawn so that every mechanism matters to the logits.  ``sharp``
     multiplies the attention's query projections: with large values a query's softmax rests on one or two keys
-    somewhere in its context, far ones as often as near ones."""
+    somewhere in its context, far ones as often as near ones.  ``apart``: the routers' corrections lie 1.5 apart,
+    more than two scores can differ, so that no choice of experts is a close call (for runs in bfloat16, whose
+    rounding would flip close calls; the scores still weigh the chosen experts)."""
     cfg = CASES[name]
     g = torch.Generator().manual_seed(seed)
     W: Dict[str, torch.Tensor] = {}
@@ -147,6 +149,8 @@ def make_weights(name: str, seed: int = 0, sharp: float = 1.0) -> Dict[str, torc
             # (corrections as large as the scores' differences: the choice and the weights then often disagree,
             # and some choice scores are negative)
             W[f"{p}.mlp.correction"] = normal(E, std=0.15, mean=-0.05)
+            if apart:
+                W[f"{p}.mlp.correction"] = (torch.randperm(E, generator=g).to(torch.float64) - E / 2) * 1.5
             for e in range(E):
                 W[f"{p}.mlp.e{e}.gate"] = normal(ff, width, std=1.5 * width ** -0.5)
                 W[f"{p}.mlp.e{e}.up"] = normal(ff, width, std=1.5 * width ** -0.5)

@@ -288,6 +288,32 @@ class EmuOps:
                 wts[t, i] = s[t, e]
         return dense, ids, wts
 
+    def moe_plan(self, ids, experts):
+        flat = ids.reshape(-1).tolist()
+        counts, rank = [0] * experts, []
+        for e in flat:
+            rank.append(counts[e])
+            counts[e] += 1
+        offsets = [0]
+        for c in counts:
+            offsets.append(offsets[-1] + c)
+        return (torch.tensor(counts, dtype=torch.int32), torch.tensor(offsets, dtype=torch.int32),
+                torch.tensor(rank, dtype=torch.int32).reshape(ids.shape))
+
+    def moe_gather(self, x, ids, rank, offsets):
+        n, top = ids.shape
+        row_of = (offsets.long()[ids.long()] + rank.long()).to(torch.int32)
+        xg = torch.zeros(n * top, x.shape[1], dtype=x.dtype)
+        xg[row_of.long().reshape(-1)] = x.repeat_interleave(top, dim=0)
+        return xg, row_of
+
+    def moe_scatter(self, yg, row_of, weights, y=None):
+        add = (weights.double()[:, :, None] * yg.double()[row_of.long()]).sum(1)
+        if y is None:
+            return add.to(torch.float32)
+        y.copy_((y.double() + add).to(torch.float32))
+        return y
+
     def moe_accumulate(self, y, part, dense, expert):
         add = dense.double()[:, expert: expert + 1] * part.double()
         if y is None:

@@ -215,7 +215,7 @@ def test_sharp_attention_over_far_keys_and_page_borders(dirs, tmp_path):
     toks = cases.tokens("pair", 150, 5)
     ref = plain.forward(cfg, W, toks)
     # the test's premise: losing the oldest keys must show (the plain implementation on a prompt without them differs)
-    assert plain.logit_error(plain.forward(cfg, W, toks[40:])[-20:], ref[-20:]) > 0.05
+    assert plain.logit_error(plain.forward(cfg, W, toks[40:])[-20:], ref[-20:]) > 0.5
     runner = _runner(folder, 192)
     runner.add_request("r")
     rows, at = [], 0
