@@ -63,6 +63,7 @@ def parse_args():
                          "beside Llama layers of equal size, with the time of every kernel entry point")
     ap.add_argument("--design-sizes", default="2048,4096", help="model widths of --design (comma separated)")
     ap.add_argument("--design-layers", type=int, default=4, help="layers of each model of --design")
+    ap.add_argument("--design-models", default="", help="which models of --design run (comma separated; empty: all)")
     return ap.parse_args()
 
 
@@ -172,7 +173,8 @@ def design_bench(args) -> int:
                   ("llama", llama_config(width, ff, heads, dim, kv, args.design_layers))]
         if design == "bomotar":
             models.insert(0, ("bomotar", bomotar_config(width, ff, heads, dim, kv, args.design_layers)))
-        for name, cfg in models:
+        chosen = [m for m in args.design_models.split(",") if m]
+        for name, cfg in [m for m in models if not chosen or m[0] in chosen]:
             say(f"{name} width {width}: building")
             model = random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
             points[f"{name}_w{width}"] = measure(model)
@@ -180,7 +182,7 @@ def design_bench(args) -> int:
                 f"decode {points[f'{name}_w{width}']['decode_tokens_per_s']} tok/s")
             del model
             torch.cuda.empty_cache()
-    first = f"{design}_w{args.design_sizes.split(',')[0]}"
+    first = next(iter(points))
     print(json.dumps({"metric": f"{design}_prefill_tokens_per_s_T{T}", "value": points[first]["prefill_tokens_per_s"], "unit": "tokens/s",
                       "n_gpus": 1, "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
                       "data": "synthetic", "vs_baseline": None,

@@ -1,7 +1,7 @@
 // A gated delta-rule mixer over a batch of requests that each bring a run of tokens: the recurrence over a
 // per-request state, the small second product of a low-rank projection with the recurrence's decay or a sigmoid in
 // its epilogue, and the per-head norm with its gate behind the recurrence.  All arithmetic is float32; the state
-// [heads, key_dim, value_dim] lives in float32 rows of a per-request state tensor (row = request slot).
+// [heads, value_dim, key_dim] lives in float32 rows of a per-request state tensor (row = request slot).
 //
 // A request r of the batch owns tokens cu_seqlens[r] .. cu_seqlens[r + 1] - 1 and the state row state_slots[r];
 // everything is read from device memory, so the same launches serve prompt portions, single decoded tokens and
@@ -110,12 +110,21 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaArgs a) {
   const bool col_ok = j < a.vdim;
   const int kvh = h / (a.heads / a.kv_heads);
 
-  float* S_mem = a.state + (size_t)a.state_slots[r] * a.state_stride + a.state_off + (size_t)h * a.dim * a.vdim;
+  // a head's state lies in memory column by column, [vdim][dim]: the key channels of one value column are
+  // neighbours, so a lane's entries are one or two 16-byte pieces and a wave's columns one contiguous run
+  float* S_mem = a.state + (size_t)a.state_slots[r] * a.state_stride + a.state_off + ((size_t)h * a.vdim + (col_ok ? j : 0)) * a.dim;
+  const bool vec = a.dim % 4 == 0 && ((uintptr_t)S_mem % 16) == 0;
   float S[PER];
 #pragma unroll
-  for (int e = 0; e < PER; ++e) {
-    const int i = ks * PER + e;
-    S[e] = (col_ok && i < a.dim) ? S_mem[(size_t)i * a.vdim + j] : 0.f;
+  for (int e4 = 0; e4 < PER / 4; ++e4) {
+    const int i = ks * PER + e4 * 4;
+    if (vec && col_ok && i < a.dim) {
+      const float4 v = *(const float4*)(S_mem + i);
+      S[e4 * 4 + 0] = v.x; S[e4 * 4 + 1] = v.y; S[e4 * 4 + 2] = v.z; S[e4 * 4 + 3] = v.w;
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) S[e4 * 4 + c] = (col_ok && i + c < a.dim) ? S_mem[i + c] : 0.f;
+    }
   }
   const int q_col = kvh * a.dim, k_col = (a.kv_heads + kvh) * a.dim, v_col = 2 * a.kv_heads * a.dim + h * a.vdim;
   const int out_width = a.heads * a.vdim;
@@ -146,6 +155,59 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaArgs a) {
       rkq = a.kq[row * a.kv_heads + kvh];
     }
   };
+  struct Tok {
+    float4 q[PER / 4], k[PER / 4], g[PER / 4];
+    float b, v, kq;
+  };
+  auto take = [&](Tok& x, int t) {
+    const float4* q4 = (const float4*)(qs + t * DP + ks * PER);
+    const float4* k4 = (const float4*)(kk + t * DP + ks * PER);
+    const float4* g4 = (const float4*)(gs + t * DP + ks * PER);
+#pragma unroll
+    for (int e4 = 0; e4 < PER / 4; ++e4) {
+      x.q[e4] = q4[e4];
+      x.k[e4] = k4[e4];
+      x.g[e4] = g4[e4];
+    }
+    x.b = bs[t];
+    x.v = vs[t * CB + jl];
+    x.kq = kqs[t];
+  };
+  auto step = [&](const Tok& x, int t_run) {
+    float pred[PER / 4], read[PER / 4];
+#pragma unroll
+    for (int e4 = 0; e4 < PER / 4; ++e4) {
+      const float qa[4] = {x.q[e4].x, x.q[e4].y, x.q[e4].z, x.q[e4].w}, ka[4] = {x.k[e4].x, x.k[e4].y, x.k[e4].z, x.k[e4].w},
+                  ga[4] = {x.g[e4].x, x.g[e4].y, x.g[e4].z, x.g[e4].w};
+      float p = 0.f, rd = 0.f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int e = e4 * 4 + c;
+        S[e] *= ga[c];
+        p = fmaf(S[e], ka[c], p);
+        rd = fmaf(S[e], qa[c], rd);
+      }
+      pred[e4] = p;
+      read[e4] = rd;
+    }
+    float ps = pred[0], rs = read[0];
+#pragma unroll
+    for (int e4 = 1; e4 < PER / 4; ++e4) {   // (a fixed order: the same sums wherever the token stands)
+      ps += pred[e4];
+      rs += read[e4];
+    }
+    ps = column_sum<KS>(ps);
+    rs = column_sum<KS>(rs);
+    const float u = x.b * (x.v - ps);
+#pragma unroll
+    for (int e4 = 0; e4 < PER / 4; ++e4) {
+      S[e4 * 4 + 0] = fmaf(x.k[e4].x, u, S[e4 * 4 + 0]);
+      S[e4 * 4 + 1] = fmaf(x.k[e4].y, u, S[e4 * 4 + 1]);
+      S[e4 * 4 + 2] = fmaf(x.k[e4].z, u, S[e4 * 4 + 2]);
+      S[e4 * 4 + 3] = fmaf(x.k[e4].w, u, S[e4 * 4 + 3]);
+    }
+    if (ks == 0 && col_ok) a.y[(size_t)(start + t_run) * out_width + (size_t)h * a.vdim + j] = fmaf(u, x.kq, rs);
+  };
   fetch(0);
   for (int t0 = 0; t0 < len; t0 += TC) {
     const int tc = min(TC, len - t0);
@@ -170,46 +232,29 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaArgs a) {
     }
     __syncthreads();
     if (t0 + TC < len) fetch(t0 + TC);   // on its way while this chunk runs
-    for (int t = 0; t < tc; ++t) {
-      const float4* q4 = (const float4*)(qs + t * DP + ks * PER);
-      const float4* k4 = (const float4*)(kk + t * DP + ks * PER);
-      const float4* g4 = (const float4*)(gs + t * DP + ks * PER);
-      float kr[PER];
-      float pred[PER / 4], read[PER / 4];
-#pragma unroll
-      for (int e4 = 0; e4 < PER / 4; ++e4) {
-        const float4 q = q4[e4], k = k4[e4], g = g4[e4];
-        const float qa[4] = {q.x, q.y, q.z, q.w}, ka[4] = {k.x, k.y, k.z, k.w}, ga[4] = {g.x, g.y, g.z, g.w};
-        float p = 0.f, rd = 0.f;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const int e = e4 * 4 + c;
-          kr[e] = ka[c];
-          S[e] *= ga[c];
-          p = fmaf(S[e], ka[c], p);
-          rd = fmaf(S[e], qa[c], rd);
-        }
-        pred[e4] = p;
-        read[e4] = rd;
+    // two tokens a turn, each token's LDS reads issued before the token ahead of it is worked on: a wave issues in
+    // order, and reads that start only when the chain reaches them would add their whole latency to every token
+    Tok A, B;
+    take(A, 0);
+    for (int t = 0; t < tc; t += 2) {
+      if (t + 1 < tc) take(B, t + 1);
+      step(A, t0 + t);
+      if (t + 1 < tc) {
+        if (t + 2 < tc) take(A, t + 2);
+        step(B, t0 + t + 1);
       }
-      float ps = pred[0], rs = read[0];
-#pragma unroll
-      for (int e4 = 1; e4 < PER / 4; ++e4) {   // (a fixed order: the same sums wherever the token stands)
-        ps += pred[e4];
-        rs += read[e4];
-      }
-      ps = column_sum<KS>(ps);
-      rs = column_sum<KS>(rs);
-      const float u = bs[t] * (vs[t * CB + jl] - ps);
-#pragma unroll
-      for (int e = 0; e < PER; ++e) S[e] = fmaf(kr[e], u, S[e]);
-      if (ks == 0 && col_ok) a.y[(size_t)(start + t0 + t) * out_width + (size_t)h * a.vdim + j] = fmaf(u, kqs[t], rs);
     }
   }
 #pragma unroll
-  for (int e = 0; e < PER; ++e) {
-    const int i = ks * PER + e;
-    if (col_ok && i < a.dim) S_mem[(size_t)i * a.vdim + j] = S[e];
+  for (int e4 = 0; e4 < PER / 4; ++e4) {
+    const int i = ks * PER + e4 * 4;
+    if (vec && col_ok && i < a.dim) {
+      *(float4*)(S_mem + i) = make_float4(S[e4 * 4 + 0], S[e4 * 4 + 1], S[e4 * 4 + 2], S[e4 * 4 + 3]);
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (col_ok && i + c < a.dim) S_mem[i + c] = S[e4 * 4 + c];
+    }
   }
 }
 
@@ -265,10 +310,11 @@ __global__ __launch_bounds__(256) void lowrank_up_kernel(const float* __restrict
                                                          const float* __restrict__ wt, float* __restrict__ out, int n,
                                                          int n_out, int mode, const float* __restrict__ a_log,
                                                          const float* __restrict__ bias, int per_head) {
+  // (blocks of 64 or 256 threads: a thread owns one column)
   extern __shared__ __attribute__((aligned(16))) float xs[];   // [LR_ROWS][rank4]: rows padded with zeros to four
   const int rank4 = (rank + 3) & ~3;
-  const int t0 = blockIdx.x * LR_ROWS, c = blockIdx.y * 256 + threadIdx.x;
-  for (int idx = threadIdx.x; idx < LR_ROWS * rank4; idx += 256) {
+  const int t0 = blockIdx.x * LR_ROWS, c = blockIdx.y * blockDim.x + threadIdx.x;
+  for (int idx = threadIdx.x; idx < LR_ROWS * rank4; idx += blockDim.x) {
     const int t = idx / rank4, i = idx % rank4;
     xs[idx] = (t0 + t < n && i < rank) ? x[(size_t)(t0 + t) * x_stride + col0 + i] : 0.f;
   }
@@ -277,6 +323,7 @@ __global__ __launch_bounds__(256) void lowrank_up_kernel(const float* __restrict
   float acc[LR_ROWS];
 #pragma unroll
   for (int t = 0; t < LR_ROWS; ++t) acc[t] = 0.f;
+#pragma unroll 4
   for (int i = 0; i < rank4; i += 4) {   // (ascending i for every row: the same sums wherever the row stands)
     float w[4];
 #pragma unroll
@@ -312,9 +359,11 @@ extern "C" int tp_lowrank_up(const float* x, int x_stride, int col0, int rank, c
   TP_REQUIRE(mode >= 0 && mode <= 2, "lowrank_up: unknown epilogue %d", mode);
   TP_REQUIRE(mode != 2 || (a_log && bias && per_head > 0), "lowrank_up: the decay needs its rates and biases");
   if (n == 0) return 0;
-  const dim3 grid((n + LR_ROWS - 1) / LR_ROWS, (n_out + 255) / 256);
+  // (a few rows: blocks of one wave, so that the columns are spread over many CUs)
+  const int threads = n <= 64 ? 64 : 256;
+  const dim3 grid((n + LR_ROWS - 1) / LR_ROWS, (n_out + threads - 1) / threads);
   TP_REQUIRE(grid.y <= 65535, "lowrank_up: too many columns");
-  hipLaunchKernelGGL(lowrank_up_kernel, grid, dim3(256), sizeof(float) * LR_ROWS * ((rank + 3) & ~3), s, x, x_stride, col0, rank, wt, out, n,
+  hipLaunchKernelGGL(lowrank_up_kernel, grid, dim3(threads), sizeof(float) * LR_ROWS * ((rank + 3) & ~3), s, x, x_stride, col0, rank, wt, out, n,
                      n_out, mode, a_log, bias, per_head);
   TP_CHECK_LAUNCH("lowrank_up");
   return 0;

@@ -1,6 +1,6 @@
 // Small kernels around the products of a layer: an embedding with a hashed bigram table, the gate on an attention's
 // output, the norm behind a sublayer added into the residual stream, a plain activation, and the router of a
-// mixture of experts with the weighted sum of its experts' outputs.  Float32 arithmetic throughout; a row's result
+// mixture of experts and what moves rows into the order of the experts and back.  Float32 arithmetic throughout; a row's result
 // never depends on other rows.
 #include <math.h>
 
@@ -159,11 +159,93 @@ __global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ h, co
   for (int c = threadIdx.x; c < width; c += blockDim.x) from_float(x + base + c, h[base + c] * rstd2 * w_next[c]);
 }
 
+// The same with the row in registers: every value is read once, sixteen bytes a load, all loads of a pass in flight
+// together (width a multiple of four, at most 256 * 4 * NV).  The sums are formed in the generic kernel's order of
+// a thread's own elements only where the widths agree; a row's result never depends on other rows either way.
+template <typename TO, int NV>
+__global__ __launch_bounds__(256) void norm_add_reg_kernel(float* __restrict__ h, const float* __restrict__ y,
+                                                           const float* __restrict__ w, float eps,
+                                                           const float* __restrict__ w_next, float eps_next,
+                                                           TO* __restrict__ x, int width) {
+  __shared__ float scratch[32];
+  const size_t base = (size_t)blockIdx.x * width;
+  const int w4 = width / 4;
+  float4 yv[NV], hv[NV], wv[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int c = k * 256 + threadIdx.x;
+    if (c < w4) {
+      yv[k] = *(const float4*)(y + base + 4 * c);
+      hv[k] = *(const float4*)(h + base + 4 * c);
+      wv[k] = *(const float4*)(w + 4 * c);
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+    if (k * 256 + threadIdx.x < w4) {
+      ss = fmaf(yv[k].x, yv[k].x, ss);
+      ss = fmaf(yv[k].y, yv[k].y, ss);
+      ss = fmaf(yv[k].z, yv[k].z, ss);
+      ss = fmaf(yv[k].w, yv[k].w, ss);
+    }
+  ss = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(ss / (float)width + eps);
+  float ss2 = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int c = k * 256 + threadIdx.x;
+    if (c < w4) {
+      hv[k].x += yv[k].x * rstd * wv[k].x;
+      hv[k].y += yv[k].y * rstd * wv[k].y;
+      hv[k].z += yv[k].z * rstd * wv[k].z;
+      hv[k].w += yv[k].w * rstd * wv[k].w;
+      *(float4*)(h + base + 4 * c) = hv[k];
+      ss2 = fmaf(hv[k].x, hv[k].x, ss2);
+      ss2 = fmaf(hv[k].y, hv[k].y, ss2);
+      ss2 = fmaf(hv[k].z, hv[k].z, ss2);
+      ss2 = fmaf(hv[k].w, hv[k].w, ss2);
+    }
+  }
+  if (w_next == nullptr) return;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int c = k * 256 + threadIdx.x;
+    if (c < w4) wv[k] = *(const float4*)(w_next + 4 * c);
+  }
+  ss2 = block_sum(ss2, scratch);
+  const float rstd2 = 1.0f / sqrtf(ss2 / (float)width + eps_next);
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int c = k * 256 + threadIdx.x;
+    if (c < w4) from_float4(x + base + 4 * c, hv[k].x * rstd2 * wv[k].x, hv[k].y * rstd2 * wv[k].y, hv[k].z * rstd2 * wv[k].z, hv[k].w * rstd2 * wv[k].w);
+  }
+}
+
 extern "C" int tp_norm_add(float* h, const float* y, const float* w, float eps, const float* w_next, float eps_next, void* x,
                            int x_dt, int n, int width, hipStream_t s) {
   TP_REQUIRE(n >= 0 && width > 0, "norm_add: bad sizes");
   TP_REQUIRE(w_next == nullptr || x != nullptr, "norm_add: no place for the next rows");
   if (n == 0) return 0;
+  TP_REQUIRE(w_next == nullptr || x_dt == TP_F32 || x_dt == TP_BF16, "norm_add: unknown dtype %d", x_dt);
+  const bool aligned = ((uintptr_t)h % 16) == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)w_next % 16) == 0 &&
+                       ((uintptr_t)x % 16) == 0;
+  if (width % 4 == 0 && width >= 1024 && width <= 256 * 4 * 8 && aligned) {
+    const bool bf = w_next != nullptr && x_dt == TP_BF16;
+#define NA(NV)                                                                                                                   \
+  do {                                                                                                                           \
+    if (bf)                                                                                                                      \
+      hipLaunchKernelGGL((norm_add_reg_kernel<bf16_t, NV>), dim3(n), dim3(256), 0, s, h, y, w, eps, w_next, eps_next, (bf16_t*)x, width); \
+    else                                                                                                                         \
+      hipLaunchKernelGGL((norm_add_reg_kernel<float, NV>), dim3(n), dim3(256), 0, s, h, y, w, eps, w_next, eps_next, (float*)x, width);   \
+  } while (0)
+    if (width <= 2048) NA(2);
+    else if (width <= 4096) NA(4);
+    else NA(8);
+#undef NA
+    TP_CHECK_LAUNCH("norm_add");
+    return 0;
+  }
   const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
   if (w_next == nullptr || x_dt == TP_F32)
     hipLaunchKernelGGL(norm_add_kernel<float>, dim3(n), dim3(threads), 0, s, h, y, w, eps, w_next, eps_next, (float*)x, width);
@@ -360,27 +442,6 @@ extern "C" int tp_moe_route(const float* logits, int logit_stride, const float* 
   return 0;
 }
 
-// y[t] += dense[t, e] * part[t]: the weighted sum of the experts' outputs, one expert after the other.
-__global__ void moe_accumulate_kernel(float* __restrict__ y, const float* __restrict__ part, const float* __restrict__ dense,
-                                      int experts, int e, int width, size_t total, int first) {
-  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= total) return;
-  const size_t t = i / width;
-  const float w = dense[t * experts + e];
-  y[i] = first ? w * part[i] : fmaf(w, part[i], y[i]);
-}
-
-extern "C" int tp_moe_accumulate(float* y, const float* part, const float* dense, int experts, int e, int n, int width, int first,
-                                 hipStream_t s) {
-  TP_REQUIRE(n >= 0 && width > 0 && e >= 0 && e < experts, "moe_accumulate: bad sizes");
-  if (n == 0) return 0;
-  const size_t total = (size_t)n * width;
-  hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, y, part, dense, experts, e,
-                     width, total, first);
-  TP_CHECK_LAUNCH("moe_accumulate");
-  return 0;
-}
-
 // ---- rows sorted by expert --------------------------------------------------------------------
 // For steps of many rows the chosen (token, expert) pairs are brought into the order of the experts, so that
 // every expert is one product over its own rows.  ids [n, top] lists each token's experts; pair p = t * top + k.
@@ -469,5 +530,34 @@ extern "C" int tp_moe_scatter(const float* yg, const int* row_of, const float* w
   if (n == 0) return 0;
   hipLaunchKernelGGL(moe_scatter_kernel, dim3(n), dim3(width >= 256 ? 256 : 64), 0, s, yg, row_of, weights, y, top, width, accumulate);
   TP_CHECK_LAUNCH("moe_scatter");
+  return 0;
+}
+
+// out[e][t][c] = a[t][e * ff + c] * dense[t][e]: the activations of all experts of a few rows, each expert's as rows
+// of its own, times the token's weight for the expert (zero where it was not chosen); formed in float32, rounded once.
+template <typename T>
+__global__ void moe_spread_kernel(const T* __restrict__ a, const float* __restrict__ dense, T* __restrict__ out, int n, int experts,
+                                  int ff, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int c = (int)(i % ff);
+  const size_t te = i / ff;
+  const int e = (int)(te % experts);
+  const size_t t = te / experts;
+  from_float(out + ((size_t)e * n + t) * ff + c, to_float(a[i]) * dense[t * experts + e]);
+}
+
+extern "C" int tp_moe_spread(const void* a, int dt, const float* dense, void* out, int n, int experts, int ff, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && experts > 0 && ff > 0, "moe_spread: bad sizes");
+  if (n == 0) return 0;
+  const size_t total = (size_t)n * experts * ff;
+  const dim3 grid((unsigned)((total + 255) / 256));
+  if (dt == TP_F32)
+    hipLaunchKernelGGL(moe_spread_kernel<float>, grid, dim3(256), 0, s, (const float*)a, dense, (float*)out, n, experts, ff, total);
+  else if (dt == TP_BF16)
+    hipLaunchKernelGGL(moe_spread_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)a, dense, (bf16_t*)out, n, experts, ff, total);
+  else
+    TP_REQUIRE(false, "moe_spread: unknown dtype %d", dt);
+  TP_CHECK_LAUNCH("moe_spread");
   return 0;
 }

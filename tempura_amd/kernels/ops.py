@@ -1278,22 +1278,6 @@ def moe_route(logits: torch.Tensor, correction: torch.Tensor, experts: int, top:
     return dense, ids, weights
 
 
-def moe_accumulate(y: Optional[torch.Tensor], part: torch.Tensor, dense: torch.Tensor, expert: int) -> torch.Tensor:
-    """y[t] += dense[t, expert] * part[t] (float32 [n, width]); ``y`` None: a new tensor holding the product."""
-    if _backend is not None:
-        return _backend.moe_accumulate(y, part, dense, expert)
-    _dev_ok(y, part, dense)
-    _need(part.dtype == torch.float32 and part.dim() == 2 and dense.dtype == torch.float32 and dense.dim() == 2
-          and dense.shape[0] == part.shape[0] and 0 <= expert < dense.shape[1], "moe_accumulate: bad operands")
-    first = y is None
-    if first:
-        y = torch.empty_like(part)
-    _need(y.dtype == torch.float32 and tuple(y.shape) == tuple(part.shape), "moe_accumulate: y must match the expert's output")
-    _call("tp_moe_accumulate", _ptr(y), _ptr(part), _ptr(dense), dense.shape[1], int(expert), part.shape[0], part.shape[1], int(first),
-          _stream())
-    return y
-
-
 LOWRANK_MODES = {"plain": 0, "sigmoid": 1, "decay": 2}
 
 
@@ -1324,7 +1308,7 @@ def delta_scan(qkv: torch.Tensor, decay: torch.Tensor, proj: torch.Tensor, beta_
     """The gated delta rule per head over each request's run.  ``qkv`` float32 [n, q | k | v] with q and k
     [kv_heads * dim] and v [heads * vdim]; q and k are made unit vectors per head (x / sqrt(sum x^2 + unit_eps), q times
     ``q_scale``); beta = sigmoid(proj[:, beta_col0 + h]); ``decay`` float32 [n, heads * dim].  Per head, with S
-    [dim, vdim] at ``state[slot, state_off:]``:  S <- decay * S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
+    [dim, vdim] (kept at ``state[slot, state_off:]`` column by column, [heads, vdim, dim]):  S <- decay * S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
     Returns o float32 [n, heads * vdim]; the state is left as the run leaves it.  (q and k of ``qkv`` are left as
     unit vectors: the rows are a temporary of the caller's.)"""
     if _backend is not None:
@@ -1407,3 +1391,18 @@ def moe_scatter(yg: torch.Tensor, row_of: torch.Tensor, weights: torch.Tensor, y
     _need(y.dtype == torch.float32 and tuple(y.shape) == (n, yg.shape[1]), "moe_scatter: y must be float32 [n, width]")
     _call("tp_moe_scatter", _ptr(yg), _ptr(row_of), _ptr(weights), _ptr(y), n, top, yg.shape[1], int(acc), _stream())
     return y
+
+
+def moe_spread(a: torch.Tensor, dense: torch.Tensor, experts: int) -> torch.Tensor:
+    """``a`` [n, experts * ff] (all experts' activations of every row) -> [experts, n, ff]: each expert's activations
+    as rows of its own, times the row's weight for the expert (``dense`` float32 [n, experts], zero where the expert
+    was not chosen); the product is formed in float32 and rounded once."""
+    if _backend is not None:
+        return _backend.moe_spread(a, dense, experts)
+    _dev_ok(a, dense)
+    _need(a.dim() == 2 and a.shape[1] % experts == 0 and dense.dtype == torch.float32 and tuple(dense.shape) == (a.shape[0], experts),
+          "moe_spread: bad operands")
+    n, ff = a.shape[0], a.shape[1] // experts
+    out = torch.empty((experts, n, ff), dtype=a.dtype, device=a.device)
+    _call("tp_moe_spread", _ptr(a), _dt(a), _ptr(dense), _ptr(out), n, int(experts), ff, _stream())
+    return out

@@ -16,7 +16,7 @@ dtype; the two low-rank second products run in float32 on the first products' fl
 
 The columns of its input product are [q | k | v | beta | a1 | g1]; the ranks of the two low-rank projections are the
 checkpoint's own.  Per request it keeps, in one float32 row, the convolution's last ``conv_taps - 1`` inputs and the
-state [H, D, Dv].
+state (a head's [D, Dv] matrix column by column: [H, Dv, D]).
 """
 from __future__ import annotations
 

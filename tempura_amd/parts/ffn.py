@@ -143,9 +143,11 @@ class RoutedExperts(FeedForward):
     ``keep``), only looks at the experts of the ``keep`` groups whose best choice score is largest; the weights are
     the chosen experts' s, not renormalised.  The output is the weighted sum of the chosen experts' outputs.
 
-    Two ways through the experts.  A step of single tokens (decoding; it may be captured): every expert runs over
-    all rows and a row's sum takes it with its weight, which is zero where the expert was not chosen; the experts
-    are added in ascending order and nothing of the batch is read on the host.  A step with portions of prompts: the
+    Two ways through the experts.  A step of single tokens (decoding; it may be captured): ONE gate/up product
+    over the stacked weights of all experts, then every expert's activations times the row's weight for it (zero
+    where the expert was not chosen; ``ops.moe_spread``), then the experts' down products one after the other into
+    one sum, ascending; nothing of the batch is read on the host, and at a few rows with several experts each
+    nearly every expert's weights are read anyway.  A step with portions of prompts: the
     chosen (token, expert) pairs are brought into the order of the experts, the host reads how many rows each expert
     has (the one wait of the layer), every expert with rows is one pair of products over its rows, and a token's
     sum adds its experts' rows in the order of its choice.  Either way a row's result does not depend on what else
@@ -188,12 +190,17 @@ class RoutedExperts(FeedForward):
         self.w_router = ops.tile_weight(pad_rows(self._to_device(get(w["router"])), 16))
         self.correction = self._to_device(get(w["correction"]), torch.float32)
         self.fused = self.dtype == torch.bfloat16 and ops.gated_layout_ok(self.intermediate_size, self.hidden_size)
-        self.w13, self.w2 = [], []
+        stack, self.w2 = [], []
         for n in range(self.experts):
             gate, up = self._to_device(get(w["gate"].format(n))), self._to_device(get(w["up"].format(n)))
-            both = ops.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], dim=0).contiguous()
-            self.w13.append(ops.tile_weight(both))
+            stack.append(ops.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], dim=0))
             self.w2.append(ops.tile_weight(self._to_device(get(w["down"].format(n)))))
+        # the gate/up weights of all experts are one matrix (decoding runs them as one product); an expert's own
+        # are rows of it, without a copy (tiled weights are cut at multiples of sixteen rows)
+        rows = 2 * self.intermediate_size
+        stacked = torch.cat(stack, dim=0).contiguous()
+        self.w13_all = ops.tile_weight(stacked) if rows % 16 == 0 else stacked
+        self.w13 = [ops.weight_rows(self.w13_all, n * rows, (n + 1) * rows) for n in range(self.experts)]
 
     def _expert(self, n, rows):
         if self.fused:
@@ -204,9 +211,15 @@ class RoutedExperts(FeedForward):
         logits = ops.linear(x, self.w_router, torch.float32)
         dense, ids, weights = ops.moe_route(logits, self.correction, self.experts, self.top, self.groups, self.keep)
         if getattr(ctx, "max_q_len", 1) <= 1:
-            y = residual      # (None: the first expert's share starts a new tensor)
+            if self.fused:
+                a = ops.linear_swiglu(x, self.w13_all)
+            else:
+                gu = ops.linear(x, self.w13_all, torch.float32)
+                a = ops.swiglu(gu.view(-1, 2 * self.intermediate_size), self.dtype).view(x.shape[0], -1)
+            parts = ops.moe_spread(a, dense, self.experts)
+            y = residual      # (None: the first expert's product starts a new tensor)
             for n in range(self.experts):
-                y = ops.moe_accumulate(y, ops.linear(self._expert(n, x), self.w2[n], torch.float32), dense, n)
+                y = ops.linear(parts[n], self.w2[n], torch.float32, residual=y) if y is not None else ops.linear(parts[n], self.w2[n], torch.float32)
             return y if residual is None else None
         counts, offsets, rank = ops.moe_plan(ids, self.experts)
         xg, row_of = ops.moe_gather(x, ids, rank, offsets)

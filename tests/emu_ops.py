@@ -314,12 +314,9 @@ class EmuOps:
         y.copy_((y.double() + add).to(torch.float32))
         return y
 
-    def moe_accumulate(self, y, part, dense, expert):
-        add = dense.double()[:, expert: expert + 1] * part.double()
-        if y is None:
-            return add.to(torch.float32)
-        y.copy_((y.double() + add).to(torch.float32))
-        return y
+    def moe_spread(self, a, dense, experts):
+        n, ff = a.shape[0], a.shape[1] // experts
+        return (a.double().reshape(n, experts, ff) * dense.double()[:, :, None]).permute(1, 0, 2).contiguous().to(a.dtype)
 
     def lowrank_up(self, x, col0, weight_t, mode="plain", a_log=None, bias=None, per_head=0):
         r = weight_t.shape[0]
@@ -350,13 +347,14 @@ class EmuOps:
             if cu[r + 1] <= cu[r]:
                 continue
             slot = int(state_slots[r])
-            S = state[slot, state_off: state_off + size].double().reshape(heads, dim, vdim)
+            # (in memory a head's state lies column by column: [heads, vdim, dim])
+            S = state[slot, state_off: state_off + size].double().reshape(heads, vdim, dim).transpose(1, 2)
             for t in range(cu[r], cu[r + 1]):
                 S = g[t][:, :, None] * S
                 u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
                 S = S + k[t][:, :, None] * u[:, None, :]
                 y[t] = torch.einsum("hdv,hd->hv", S, q[t])
-            state[slot, state_off: state_off + size] = S.reshape(-1).to(torch.float32)
+            state[slot, state_off: state_off + size] = S.transpose(1, 2).reshape(-1).to(torch.float32)
         return y.reshape(n, heads * vdim).to(torch.float32)
 
     def head_norm_gate(self, o, weight, gate, eps, scale, heads, out, out_col0):

@@ -14,9 +14,9 @@ from emu_ops import EmuOps
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 # plain.logit_error of a whole model: the largest difference of any logit, in units of the logits' spread.  bfloat16
-# rounding alone reaches 0.05 in these small models; a lost key, a wrong state or another choice of experts costs
+# rounding alone reaches 0.1 in these small models; a lost key, a wrong state or another choice of experts costs
 # 0.3 and more (the tests that plant something check that their own premise does)
-TOL = {"float32": 1e-4, "bfloat16": 1e-1}
+TOL = {"float32": 1e-4, "bfloat16": 1.5e-1}
 emu = EmuOps()
 
 
@@ -204,16 +204,16 @@ def test_router_chooses_by_corrected_scores_within_the_best_groups(E, top, group
     assert int((dense > 0).sum()) == n * top
 
 
-def test_experts_outputs_add_up_with_their_weights():
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_experts_activations_as_rows_of_their_own_times_the_weights(dtype):
     ops = _ops()
     g = torch.Generator().manual_seed(4)
-    dense = torch.rand(19, 5, generator=g) * (torch.rand(19, 5, generator=g) > 0.5)
-    y_dev = y_ref = None
-    for e in range(5):
-        part = torch.randn(19, 70, generator=g)
-        y_dev = ops.moe_accumulate(y_dev, part.to(DEV), dense.to(DEV), e)
-        y_ref = emu.moe_accumulate(y_ref, part, dense, e)
-    _close(y_dev, y_ref, 1e-6)
+    n, E, ff = 19, 5, 24
+    dense = torch.rand(n, E, generator=g) * (torch.rand(n, E, generator=g) > 0.5)
+    a = torch.randn(n, E * ff, generator=g).to(dtype)
+    got = ops.moe_spread(a.to(DEV), dense.to(DEV), E)
+    assert got.shape == (E, n, ff)
+    _close(got, emu.moe_spread(a, dense, E), 1e-6 if dtype == torch.float32 else 8e-3)
 
 
 @pytest.mark.parametrize("n,top,E,width,dtype", [(77, 2, 6, 48, torch.float32), (1000, 4, 8, 64, torch.bfloat16), (5, 1, 4, 32, torch.bfloat16),
