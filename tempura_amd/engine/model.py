@@ -116,16 +116,25 @@ class CausalLM:
 
         def add(t):
             nonlocal total
+            if isinstance(t, (list, tuple)):      # (a part may keep a list of weights: one per expert)
+                for u in t:
+                    add(u)
+                return
             if isinstance(t, ops.TiledWeight):
                 t = t.data
-            if isinstance(t, torch.Tensor) and t.data_ptr() not in seen:
-                seen.add(t.data_ptr())
-                total += t.numel() * t.element_size()
+            if isinstance(t, torch.Tensor):
+                # by storage: a weight that is rows of another (no copy) counts once
+                store = t.untyped_storage()
+                if store.data_ptr() not in seen:
+                    seen.add(store.data_ptr())
+                    total += store.nbytes()
         objs = [self.final_norm, self.lm_head]
         if include_embedding:
             objs.append(self.embedding)
         for layer in self.layers:
-            objs.extend(layer.parts())
+            for part in layer.parts():
+                objs.append(part)
+                objs.extend(getattr(part, "branches", []))      # (a mixer of several mixers)
         for o in objs:
             for v in vars(o).values():
                 add(v)
