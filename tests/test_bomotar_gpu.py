@@ -163,7 +163,7 @@ def test_gate_on_the_heads_into_a_wider_buffer(dtype):
     assert torch.equal(dev.cpu()[:, :3], out[:, :3])
 
 
-@pytest.mark.parametrize("width", [48, 256, 1000, 5000])
+@pytest.mark.parametrize("width", [48, 256, 1000, 1024, 2048, 4096, 5000, 8192, 8196])
 @pytest.mark.parametrize("out_dtype", [None, torch.float32, torch.bfloat16])
 def test_norm_of_a_sublayers_output_into_the_stream(width, out_dtype):
     ops = _ops()
