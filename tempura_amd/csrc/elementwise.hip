@@ -150,7 +150,7 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
                                      int n_heads, int n_kv, int head_dim, TQ* __restrict__ q_out,
                                      TC* __restrict__ k_cache, TC* __restrict__ v_cache, int page_size,
                                      int pairs, int heads_per_block, int splits, size_t split_stride,
-                                     const float2* __restrict__ cos_sin, int with_values) {
+                                     const float2* __restrict__ cos_sin, int with_values, int out_dim) {
   const int t = blockIdx.x;
   const int hl = threadIdx.x / pairs, d = threadIdx.x % pairs;   // pairs = head_dim / 2
   const int h = blockIdx.y * heads_per_block + hl;
@@ -196,14 +196,23 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
     y0 = x0 * c - x1 * sn;
     y1 = x0 * sn + x1 * c;
   }
+  // (out_dim > head_dim: q and k leave as heads of out_dim elements, zeros behind the head's own)
   if (h < n_heads) {
-    TQ* o = q_out + ((size_t)t * n_heads + h) * head_dim;
+    TQ* o = q_out + ((size_t)t * n_heads + h) * out_dim;
     from_float(o + i0, y0);
     from_float(o + i1, y1);
+    for (int z = head_dim + 2 * d; z < out_dim; z += head_dim) {
+      from_float(o + z, 0.f);
+      from_float(o + z + 1, 0.f);
+    }
   } else if (h < n_heads + n_kv) {
-    TC* o = k_cache + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
+    TC* o = k_cache + ((page * n_kv + (h - n_heads)) * page_size + off) * out_dim;
     from_float(o + i0, y0);
     from_float(o + i1, y1);
+    for (int z = head_dim + 2 * d; z < out_dim; z += head_dim) {
+      from_float(o + z, 0.f);
+      from_float(o + z + 1, 0.f);
+    }
   } else {
     TC* o = v_cache + ((page * n_kv + (h - n_heads - n_kv)) * head_dim) * page_size + off;
     from_float(o + (size_t)i0 * page_size, y0);
@@ -234,7 +243,7 @@ __global__ void rope_qk4_kernel(const float* __restrict__ qkv, int row_stride, c
                                 const int* __restrict__ slots, const double* __restrict__ inv_freq, int rotary_dim,
                                 float factor, int n_heads, int n_rot_heads, int n_kv, int head_dim,
                                 TQ* __restrict__ q_out, TC* __restrict__ k_cache, int page_size, int splits,
-                                size_t split_stride, const float2* __restrict__ cos_sin) {
+                                size_t split_stride, const float2* __restrict__ cos_sin, int out_dim) {
   const int t = blockIdx.x;
   const int tph = head_dim / 8;                       // threads per head
   const int idx = blockIdx.y * blockDim.x + threadIdx.x;
@@ -279,16 +288,25 @@ __global__ void rope_qk4_kernel(const float* __restrict__ qkv, int row_stride, c
       r1 = x0 * sn + x1 * c;
     }
   }
+  const float zero[4] = {0.f, 0.f, 0.f, 0.f};
   if (h < n_heads) {
-    TQ* o = q_out + ((size_t)t * n_heads + h) * head_dim;
+    TQ* o = q_out + ((size_t)t * n_heads + h) * out_dim;
     store4(o + i0, a);
     store4(o + i1, b);
+    for (int z = head_dim + 8 * j; z < out_dim; z += head_dim) {   // (zeros behind the head's own elements)
+      store4(o + z, zero);
+      store4(o + z + 4, zero);
+    }
   } else {
     const int slot = slots[t];
     const size_t page = (size_t)(slot / page_size), off = (size_t)(slot % page_size);
-    TC* o = k_cache + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
+    TC* o = k_cache + ((page * n_kv + (h - n_heads)) * page_size + off) * out_dim;
     store4(o + i0, a);
     store4(o + i1, b);
+    for (int z = head_dim + 8 * j; z < out_dim; z += head_dim) {
+      store4(o + z, zero);
+      store4(o + z + 4, zero);
+    }
   }
 }
 
@@ -354,9 +372,12 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
                                 const double* inv_freq, int rotary_dim, float factor, int n, int n_heads,
                                 int n_kv, int head_dim, void* q_out, int q_dt, void* k_cache, void* v_cache,
                                 int cache_dt, int page_size, int splits, const float* cos_sin, int value_dim,
-                                hipStream_t s) {
-  // value_dim: the size of a value head (0: head_dim); the value cache is [page, kv_head, value_dim, page_size]
+                                int out_dim, hipStream_t s) {
+  // value_dim: the size of a value head (0: head_dim); the value cache is [page, kv_head, value_dim, page_size].
+  // out_dim: the size of a head of q_out and of the key cache (0: head_dim); larger: zeros behind the head's elements.
   if (value_dim <= 0) value_dim = head_dim;
+  if (out_dim <= 0) out_dim = head_dim;
+  TP_REQUIRE(out_dim >= head_dim && out_dim % 2 == 0, "rope_kv_write: padded head size %d below head_dim %d or odd", out_dim, head_dim);
   TP_REQUIRE(n >= 0 && n_heads > 0 && n_kv >= 0 && head_dim > 0, "rope_kv_write: bad sizes");
   TP_REQUIRE(value_dim <= 1024, "rope_kv_write: value size %d exceeds 1024", value_dim);
   TP_REQUIRE(splits >= 1 && splits <= 16, "rope_kv_write: bad number of partial sums");
@@ -374,13 +395,13 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
   // long steps (prompt portions, mostly) write their values sixteen tokens at a time (value_write_kernel);
   // a batch of single decoded tokens has no runs, and a second kernel would only cost it a launch
   // (values of another size than the keys always go through it: the rotation kernel walks heads of head_dim)
-  const bool grouped_values = slots != nullptr && (n >= 256 || value_dim != head_dim) && n_kv <= 65535;
-  TP_REQUIRE(slots == nullptr || value_dim == head_dim || grouped_values, "rope_kv_write: too many key heads");
+  const bool grouped_values = slots != nullptr && (n >= 256 || value_dim != head_dim || out_dim != head_dim) && n_kv <= 65535;
+  TP_REQUIRE(slots == nullptr || (value_dim == head_dim && out_dim == head_dim) || grouped_values, "rope_kv_write: too many key heads");
   const int total_heads = n_heads + (slots ? (grouped_values ? 1 : 2) * n_kv : 0);
   const dim3 grid(n, (total_heads + hpb - 1) / hpb);
   TP_REQUIRE(grid.y <= 65535, "rope_kv_write: too many heads");
   // long steps: q and k four pairs per thread, v sixteen tokens per thread
-  if (n >= 256 && head_dim % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 4 == 0 && (slots == nullptr || grouped_values) &&
+  if (n >= 256 && head_dim % 8 == 0 && out_dim % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 4 == 0 && (slots == nullptr || grouped_values) &&
       ((uintptr_t)qkv % 16) == 0 && (split_stride % 4) == 0) {
     const int n_rot_heads = n_heads + (slots ? n_kv : 0);
     const int work = n_rot_heads * (head_dim / 8);
@@ -389,7 +410,7 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
 #define LAUNCH4(TQ, TC)                                                                                               \
   hipLaunchKernelGGL((rope_qk4_kernel<TQ, TC>), g4, dim3(256), 0, s, qkv, row_stride, positions, slots, inv_freq,      \
                      rotary_dim, factor, n_heads, n_rot_heads, n_kv, head_dim, (TQ*)q_out, (TC*)k_cache, page_size, \
-                     splits, split_stride, (const float2*)cos_sin)
+                     splits, split_stride, (const float2*)cos_sin, out_dim)
     if (q_dt == TP_F32 && cache_dt == TP_F32)
       LAUNCH4(float, float);
     else if (q_dt == TP_BF16 && cache_dt == TP_BF16)
@@ -405,7 +426,7 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
 #define LAUNCH(TQ, TC)                                                                                    \
   hipLaunchKernelGGL((rope_kv_write_kernel<TQ, TC>), grid, dim3(threads), 0, s, qkv, row_stride, positions, \
                      slots, inv_freq, rotary_dim, factor, n_heads, n_kv, head_dim, (TQ*)q_out, (TC*)k_cache, \
-                     (TC*)v_cache, page_size, pairs, hpb, splits, split_stride, (const float2*)cos_sin, grouped_values ? 0 : 1)
+                     (TC*)v_cache, page_size, pairs, hpb, splits, split_stride, (const float2*)cos_sin, grouped_values ? 0 : 1, out_dim)
   if (q_dt == TP_F32 && cache_dt == TP_F32)
     LAUNCH(float, float);
   else if (q_dt == TP_BF16 && cache_dt == TP_BF16)

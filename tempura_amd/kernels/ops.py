@@ -734,20 +734,24 @@ def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
                   inv_freq: Optional[torch.Tensor], rotary_dim: int, factor: float, num_heads: int,
                   num_kv_heads: int, head_dim: int, k_cache: Optional[torch.Tensor],
                   v_cache: Optional[torch.Tensor], q_dtype: torch.dtype,
-                  cos_sin: Optional[torch.Tensor] = None, value_dim: Optional[int] = None) -> torch.Tensor:
+                  cos_sin: Optional[torch.Tensor] = None, value_dim: Optional[int] = None,
+                  pad_dim: Optional[int] = None) -> torch.Tensor:
     """Rotate q and k of float32 rows [n, (heads + 2 kv_heads) * head_dim] (or the ``Partials`` of the
     projection that makes them), store k and v into the cache rows ``slots`` and return q as q_dtype
     [n, heads, head_dim].  With ``slots`` None the rows hold q only and nothing is stored.
     ``value_dim``: the size of a value head when it is not head_dim (the rows are then
     [n, (heads + kv_heads) * head_dim + kv_heads * value_dim], the value cache [pages, kv_heads, value_dim, page_size]).
+    ``pad_dim`` (>= head_dim): q comes back as [n, heads, pad_dim] and the key cache has heads of pad_dim, zeros
+    behind each head's own elements (scores are unchanged; attention kernels that want keys as wide as values then serve).
     The q and k heads are in PAIRED order: elements (2 d, 2 d + 1) of a head rotate together by the angle
     of pair d (they are elements (d, d + rotary_dim / 2) of the split-half order).
     ``cos_sin``: this step's table from ``rope_table`` (the same values, computed once for all layers)."""
     vd = head_dim if value_dim is None else int(value_dim)
+    od = head_dim if pad_dim is None else int(pad_dim)
     if _backend is not None:
-        if vd != head_dim:
+        if vd != head_dim or od != head_dim:
             return _backend.rope_kv_write(qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads,
-                                          num_kv_heads, head_dim, k_cache, v_cache, q_dtype, value_dim=vd)
+                                          num_kv_heads, head_dim, k_cache, v_cache, q_dtype, value_dim=vd, pad_dim=od)
         return _backend.rope_kv_write(qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads,
                                       num_kv_heads, head_dim, k_cache, v_cache, q_dtype)
     splits = 1
@@ -767,7 +771,7 @@ def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
         _need(k_cache is not None and v_cache is not None and k_cache.dim() == 4 and v_cache.dim() == 4
               and tuple(v_cache.shape) == (k_cache.shape[0], k_cache.shape[1], vd, k_cache.shape[2]),
               "rope_kv_write: caches must be k [pages, kv_heads, page_size, head_dim], v [pages, kv_heads, value_dim, page_size]")
-        _need(k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == head_dim, "rope_kv_write: cache layout mismatch")
+        _need(k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == od, "rope_kv_write: cache layout mismatch")
         _need(k_cache.dtype == v_cache.dtype, "rope_kv_write: cache dtypes differ")
         page_size, cache_dt = k_cache.shape[2], _dt(k_cache)
     if rotary_dim:
@@ -776,10 +780,11 @@ def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
     if cos_sin is not None:
         _need(cos_sin.is_cuda and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous()
               and tuple(cos_sin.shape) == (n, rotary_dim // 2, 2), "rope_kv_write: table must be float32 [n, rotary_dim / 2, 2]")
-    q = torch.empty((n, num_heads, head_dim), dtype=q_dtype, device=qkv.device)
+    _need(od >= head_dim and od % 2 == 0, "rope_kv_write: pad_dim must be even and at least head_dim")
+    q = torch.empty((n, num_heads, od), dtype=q_dtype, device=qkv.device)
     _call("tp_rope_kv_write", _ptr(qkv), qkv.shape[1], _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
           ctypes.c_float(factor), n, num_heads, num_kv_heads, head_dim, _ptr(q), _dtcode(q_dtype),
-          _ptr(k_cache), _ptr(v_cache), cache_dt, page_size, splits, _ptr(cos_sin), vd, _stream())
+          _ptr(k_cache), _ptr(v_cache), cache_dt, page_size, splits, _ptr(cos_sin), vd, od, _stream())
     return q
 
 

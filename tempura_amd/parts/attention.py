@@ -266,6 +266,12 @@ class ConvAttention(BranchMixer):
         self.v_dim = self.num_kv_heads * self.value_dim
         self.channels = self.q_dim + self.k_dim + self.v_dim
         self.inner = self.num_heads * self.value_dim
+        # values wider than keys, of a size the matrix-core attention kernels take: q and the cached keys get zeros
+        # behind their own elements up to the values' size (no score changes; the key pages are that much wider),
+        # so that those kernels serve; every other pair of sizes runs the general kernel
+        self.key_dim = self.head_dim
+        if dtype == torch.bfloat16 and self.head_dim < self.value_dim <= 128 and self.value_dim % 32 == 0 and self.head_dim % 2 == 0:
+            self.key_dim = self.value_dim
         self.conv_w = None
 
     @classmethod
@@ -290,9 +296,9 @@ class ConvAttention(BranchMixer):
 
     def cache_spec(self):
         kind = "window" if self.window is not None else "full"
-        if self.value_dim == self.head_dim:
-            return CacheSpec(kind, self.num_kv_heads, self.head_dim, self.window)
-        return SizedValueCacheSpec(kind, self.num_kv_heads, self.head_dim, self.window, self.value_dim)
+        if self.value_dim == self.key_dim:
+            return CacheSpec(kind, self.num_kv_heads, self.key_dim, self.window)
+        return SizedValueCacheSpec(kind, self.num_kv_heads, self.key_dim, self.window, self.value_dim)
 
     def _paired(self, t: torch.Tensor) -> torch.Tensor:
         """Rows of a q or k tensor (projection or convolution) with every head's rotary elements in paired order
@@ -327,7 +333,8 @@ class ConvAttention(BranchMixer):
             inv_freq, rotary_dim, factor = rot
             table = self.position.table(ctx) if hasattr(self.position, "table") else None
         q = ops.rope_kv_write(qkv, ctx.positions, ctx.slot_mapping[cache.group], inv_freq, rotary_dim, factor, self.num_heads,
-                              self.num_kv_heads, self.head_dim, cache.k, cache.v, self.dtype, table, value_dim=self.value_dim)
+                              self.num_kv_heads, self.head_dim, cache.k, cache.v, self.dtype, table, value_dim=self.value_dim,
+                              pad_dim=self.key_dim)
         a = ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
                                 ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len, ctx.num_single)
         ops.sigmoid_gate(a, proj if self.gate else None, col0 + self.channels, scale, out, out_col0)

@@ -178,7 +178,7 @@ class EmuOps:
         return out
 
     def rope_kv_write(self, qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads, num_kv_heads,
-                      head_dim, k_cache, v_cache, q_dtype, value_dim=None):
+                      head_dim, k_cache, v_cache, q_dtype, value_dim=None, pad_dim=None):
         n = qkv.shape[0]
         nrot = num_heads + (num_kv_heads if slots is not None else 0)
         x = qkv.double()[:, : nrot * head_dim].reshape(n, nrot, head_dim).clone()
@@ -191,6 +191,8 @@ class EmuOps:
             x0, x1 = x[..., 0:rotary_dim:2].clone(), x[..., 1:rotary_dim:2].clone()
             x[..., 0:rotary_dim:2] = x0 * c - x1 * s
             x[..., 1:rotary_dim:2] = x0 * s + x1 * c
+        if pad_dim is not None and pad_dim > head_dim:      # zeros behind every head's own elements
+            x = torch.nn.functional.pad(x, (0, pad_dim - head_dim))
         q = x[:, :num_heads].to(q_dtype).contiguous()
         if slots is not None:
             k = x[:, num_heads:]

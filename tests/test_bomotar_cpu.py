@@ -129,6 +129,12 @@ def test_router_stand_in_is_the_plain_router():
         assert int((dense > 0).sum()) == 40 * top
 
 
+@pytest.mark.parametrize("name", ["pair", "solo"])
+def test_each_part_alone_matches_its_plain_function(dirs, name):
+    import bomotar_mechanisms
+    bomotar_mechanisms.check(dirs[name], name, "cpu", TOL)
+
+
 # ---- the model through the step function --------------------------------------------------------
 @pytest.mark.parametrize("name", ["pair", "solo"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])

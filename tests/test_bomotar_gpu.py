@@ -105,18 +105,21 @@ def test_causal_conv_without_activation_at_an_offset_of_the_state(channels, taps
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,kvh,d,vd,ps,rd", [(4, 2, 16, 24, 16, 8), (3, 3, 10, 6, 8, 10), (6, 3, 64, 128, 16, 64), (2, 1, 32, 64, 32, 0), (2, 2, 8, 8, 16, 4)])
+@pytest.mark.parametrize("heads,kvh,d,vd,ps,rd,pad", [(4, 2, 16, 24, 16, 8, 0), (3, 3, 10, 6, 8, 10, 0), (6, 3, 64, 128, 16, 64, 0), (2, 1, 32, 64, 32, 0, 0),
+                                                      (2, 2, 8, 8, 16, 4, 0), (6, 3, 64, 128, 16, 64, 128), (4, 1, 32, 64, 16, 16, 64), (2, 2, 16, 96, 16, 8, 96),
+                                                      (3, 1, 10, 32, 8, 6, 32)])
 @pytest.mark.parametrize("n", [21, 300])
-def test_values_of_another_size_into_the_cache_and_out_of_it(dtype, heads, kvh, d, vd, ps, rd, n):
+def test_values_of_another_size_into_the_cache_and_out_of_it(dtype, heads, kvh, d, vd, ps, rd, pad, n):
     """Rotation and cache write with values wider or narrower than keys, then attention over them with one far key
-    that stands out: the first rows attend from a context of 40 tokens whose third key matches every query."""
+    that stands out: the first rows attend from a context of 40 tokens whose third key matches every query.  ``pad``:
+    q and the cached keys as wide as the values, zeros behind their own elements (the matrix-core kernels then serve)."""
     ops = _ops()
     g = torch.Generator().manual_seed(heads * 100 + d + n)
     ctx0 = 40
     total = ctx0 + n
     pages = (total + ps - 1) // ps
     order = torch.randperm(pages + 3, generator=g)[:pages].to(torch.int32)
-    kc, vc = torch.zeros(pages + 4, kvh, ps, d, dtype=dtype), torch.zeros(pages + 4, kvh, vd, ps, dtype=dtype)
+    kc, vc = torch.zeros(pages + 4, kvh, ps, pad or d, dtype=dtype), torch.zeros(pages + 4, kvh, vd, ps, dtype=dtype)
     inv = torch.pow(torch.tensor(10000.0, dtype=torch.float64), -2.0 * torch.arange(rd // 2, dtype=torch.float64) / max(rd, 1)) if rd else None
     kd, vdv = kc.to(DEV), vc.to(DEV)
     qs = []
@@ -127,8 +130,9 @@ def test_values_of_another_size_into_the_cache_and_out_of_it(dtype, heads, kvh, 
         pos = torch.arange(lo, lo + cnt, dtype=torch.int32)
         slots = torch.tensor([int(order[p // ps]) * ps + p % ps for p in range(lo, lo + cnt)], dtype=torch.int32)
         q = ops.rope_kv_write(rows.to(DEV), pos.to(DEV), slots.to(DEV), None if inv is None else inv.to(DEV), rd, 1.25, heads, kvh, d,
-                              kd, vdv, dtype, value_dim=vd)
-        qr = emu.rope_kv_write(rows, pos, slots, inv, rd, 1.25, heads, kvh, d, kc, vc, dtype, value_dim=vd)
+                              kd, vdv, dtype, value_dim=vd, pad_dim=pad or None)
+        qr = emu.rope_kv_write(rows, pos, slots, inv, rd, 1.25, heads, kvh, d, kc, vc, dtype, value_dim=vd, pad_dim=pad or None)
+        assert q.shape == (cnt, heads, pad or d)
         tol = 2e-6 if dtype == torch.float32 else 1e-2
         _close(q, qr, tol)
         qs.append(qr)
@@ -334,6 +338,12 @@ def _ref(name, rid, dtype):
     if key not in _REFS:
         _REFS[key] = plain.forward(cases.config_json(name), cases.make_weights(name, apart=key[2]), cases.requests(name)[rid])
     return _REFS[key]
+
+
+@pytest.mark.parametrize("name", ["pair", "solo", "wide"])
+def test_each_part_alone_matches_its_plain_function(dirs, name):
+    import bomotar_mechanisms
+    bomotar_mechanisms.check(dirs[name], name, DEV, 2e-5)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
