@@ -107,14 +107,14 @@ def design_bench(args) -> int:
 
     def bomotar_config(width, ff, heads, dim, kv, layers):
         left = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "conv": 4, "scale": dim ** -0.5,
-                "rot": {"dims": dim, "base": 250000.0, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+                "rot": {"dims": dim, "base": 1000000.0, "scaling": {"factor": 4.0, "original": 2048, "fast": 16.0, "slow": 2.0}}}
         right = {"heads": width // 128, "kv_heads": width // 128, "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 64, "gate_rank": 64}
-        mixer = {"left": left, "right": right, "left_scale": 0.6, "right_scale": 0.9}
+        mixer = {"left": left, "right": right, "left_scale": 0.75, "right_scale": 1.1}
         dense = {"kind": "dense", "ff": ff}
         moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
         ls = [{"type": "parallel", "mixer": mixer, "mlp": moe if i % 2 else dense} for i in range(layers)]
-        return BomotarConfig.from_dict({"architecture": "Bomotar", "vocab": vocab, "width": width, "residual_mult": 0.5,
-                                        "norm": {"eps": 1e-6}, "embedding": {"bigram": {"buckets": 65521, "mul_prev": 127, "mul_cur": 17}},
+        return BomotarConfig.from_dict({"architecture": "Bomotar", "vocab": vocab, "width": width, "residual_mult": 0.8,
+                                        "norm": {"eps": 1e-6}, "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
                                         "layers": ls, "max_positions": 8192})
 
     def llama_config(width, ff, heads, dim, kv, layers):

@@ -55,9 +55,9 @@ _PB = (_left(3, 3, 10, 6, 2, rot_dims=10, base=300.0), _right(2, 1, 20, 18, 4, 9
 CASES: Dict[str, dict] = {
     # two kinds of layers, each run twice (the second time with a cache and state of its own), a layer without a
     # feed-forward between them; partial rotation with scaling; values wider than keys; grouped key heads
-    "pair": _case(70, 48, [_layer(*_PA, _dense(80), 0.6, 1.3),
+    "pair": _case(70, 48, [_layer(*_PA, _dense(80), 0.55, 1.3),
                            _layer(*_PB, _moe(24, 6, 2, (3, 2)), 1.1, 0.8),
-                           _layer(*_PA, _dense(80), 0.6, 1.3, weights_of=0),
+                           _layer(*_PA, _dense(80), 0.55, 1.3, weights_of=0),
                            _layer(_left(2, 1, 8, 8, 5), _right(3, 3, 6, 14, 1, 4, 4), None, 0.9, 0.7),
                            _layer(*_PB, _moe(24, 6, 2, (3, 2)), 1.1, 0.8, weights_of=1)], 53, 31, 7, mult=0.7, eps=1e-5),
     # one layer kind, no residual constant, no groups, one expert a token, one tap on the left (no carried
@@ -66,12 +66,12 @@ CASES: Dict[str, dict] = {
                            _layer(_left(4, 1, 6, 12, 4), _right(2, 2, 7, 5, 3, 3, 2), _dense(44))], 17, 3, 5),
     # sizes the matrix-core kernels take: heads of 64 with values of 64, heads of 32 with values of 64, a recurrence
     # with keys of 64 and of 128, eight experts in four groups
-    "wide": _case(96, 128, [_layer(_left(4, 2, 64, 64, 4, rot_dims=32, base=250000.0, scaling=(8.0, 128, 16.0, 1.0), scale=0.125),
-                                   _right(4, 2, 64, 32, 3, 16, 16), _dense(256), 0.7, 0.9),
+    "wide": _case(96, 128, [_layer(_left(4, 2, 64, 64, 4, rot_dims=32, base=500000.0, scaling=(6.0, 128, 16.0, 2.0), scale=0.11),
+                                   _right(4, 2, 64, 32, 3, 16, 16), _dense(256), 0.7, 0.85),
                             _layer(_left(2, 1, 32, 64, 3, rot_dims=32, base=10000.0), _right(2, 2, 128, 48, 4, 8, 24),
                                    _moe(64, 8, 3, (4, 2)), 1.0, 0.5),
-                            _layer(_left(4, 2, 64, 64, 4, rot_dims=32, base=250000.0, scaling=(8.0, 128, 16.0, 1.0), scale=0.125),
-                                   _right(4, 2, 64, 32, 3, 16, 16), _dense(256), 0.7, 0.9, weights_of=0)], 211, 13, 29, mult=0.5),
+                            _layer(_left(4, 2, 64, 64, 4, rot_dims=32, base=500000.0, scaling=(6.0, 128, 16.0, 2.0), scale=0.11),
+                                   _right(4, 2, 64, 32, 3, 16, 16), _dense(256), 0.7, 0.85, weights_of=0)], 211, 13, 29, mult=0.6),
 }
 
 

@@ -105,7 +105,7 @@ def test_a_layer_run_twice_has_a_cache_and_a_state_of_its_own(dirs):
 # ---- mechanisms alone, against the plain functions ----------------------------------------------
 def test_yarn_frequencies_are_the_plain_ones():
     from tempura_amd.parts.rope import rotary_inv_freq
-    for dims, base, sc in [(8, 5000.0, (4.0, 64, 8.0, 1.0)), (64, 250000.0, (8.0, 1024, 32.0, 1.0)), (32, 10000.0, (2.0, 4096, 4.0, 0.5)),
+    for dims, base, sc in [(8, 5000.0, (4.0, 64, 8.0, 1.0)), (64, 800000.0, (5.0, 2048, 24.0, 2.0)), (32, 10000.0, (2.0, 4096, 4.0, 0.5)),
                            (16, 100.0, (16.0, 8, 2.0, 1.0)), (10, 300.0, None)]:
         scaling = None if sc is None else dict(zip(("factor", "original", "fast", "slow"), sc))
         want, _ = plain.yarn_frequencies(dims, base, scaling)
