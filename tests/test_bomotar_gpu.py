@@ -370,7 +370,9 @@ def test_every_cutting_matches_plain(dirs, name, mode, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_cutting_changes_rounding_only(dirs, dtype):
-    """The same request whole, in portions and beside others: differences far below the distance to the plain result."""
+    """The same request whole, in portions and beside others: float32 differs in summation order only; bfloat16 runs
+    differ by what their roundings differ (other product kernels for other row counts, the routed feed-forward's
+    two ways), which stays at half of what a bfloat16 run may differ from the exact result."""
     reqs = cases.requests("wide")
     lengths = cases.LENGTHS["wide"]
     runs = []
@@ -379,7 +381,7 @@ def test_cutting_changes_rounding_only(dirs, dtype):
         runs.append(helpers.run_schedule(_runner(dirs.get("wide", dtype), dtype, 448), reqs, steps))
     for rid in reqs:
         for other in runs[1:]:
-            assert plain.logit_error(other[rid], runs[0][rid]) < (2e-5 if dtype == "float32" else 2e-2), rid
+            assert plain.logit_error(other[rid], runs[0][rid]) < (2e-5 if dtype == "float32" else TOL["bfloat16"] / 2), rid
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -388,14 +390,15 @@ def test_sharp_attention_over_far_keys_on_the_gpu(tmp_path, dtype):
     prompt of 400 tokens whole, then in portions that end at and beside page borders with decoding behind them."""
     from tempura_amd.engine.runner import StepEntry
     cfg = cases.config_json("wide")
-    W = cases.make_weights("wide", sharp=6.0, apart=dtype == "bfloat16")
+    # (bfloat16: scores as large as the queries carry rounding errors as large, so the queries are 2.5 instead of 6
+    # times the drawn ones and the bound is a fifth of what losing the oldest keys costs)
+    W = cases.make_weights("wide", sharp=6.0 if dtype == "float32" else 2.5, apart=dtype == "bfloat16")
     folder = cases.write_model("wide", str(tmp_path / "sharp"), weights=W)
     toks = cases.tokens("wide", 400, 5)
     ref = plain.forward(cfg, W, toks)
-    # (what losing the oldest keys costs: the premise, and for bfloat16, whose rounded scores are as large as the
-    # queries, the scale of the tolerance)
-    assert plain.logit_error(plain.forward(cfg, W, toks[200:])[-50:], ref[-50:]) > 1.2
-    tol = TOL[dtype] if dtype == "float32" else 0.4
+    # (the premise: what losing the oldest keys costs)
+    assert plain.logit_error(plain.forward(cfg, W, toks[200:])[-50:], ref[-50:]) > 1.5
+    tol = TOL[dtype] if dtype == "float32" else 0.3
     runner = _runner(folder, dtype, 448 + 448)
     runner.add_request("w")
     whole = runner.step([StepEntry("w", toks, list(range(400)))]).cpu()
