@@ -51,6 +51,9 @@ def _case(vocab, width, layers, buckets, mp, mc, mult=None, eps=1e-6):
 _PA = (_left(4, 2, 16, 24, 3, rot_dims=8, base=5000.0, scaling=(4.0, 64, 8.0, 1.0), scale=0.3), _right(4, 2, 12, 10, 2, 5, 7))
 _PB = (_left(3, 3, 10, 6, 2, rot_dims=10, base=300.0), _right(2, 1, 20, 18, 4, 9, 3))
 
+_MA = (_left(8, 2, 48, 96, 2, rot_dims=24, base=1e5, scaling=(3.0, 256, 8.0, 1.0), scale=0.2), _right(6, 3, 80, 40, 5, 12, 20))
+_MB = (_left(4, 4, 32, 32, 3, rot_dims=32, base=2e4), _right(4, 1, 48, 96, 2, 6, 10))
+
 #: name -> config.json content ("_ranks": ranks of the right mixer's low-rank projections, sizes only the tensors say)
 CASES: Dict[str, dict] = {
     # two kinds of layers, each run twice (the second time with a cache and state of its own), a layer without a
@@ -72,6 +75,13 @@ CASES: Dict[str, dict] = {
                                    _moe(64, 8, 3, (4, 2)), 1.0, 0.5),
                             _layer(_left(4, 2, 64, 64, 4, rot_dims=32, base=500000.0, scaling=(6.0, 128, 16.0, 2.0), scale=0.11),
                                    _right(4, 2, 64, 32, 3, 16, 16), _dense(256), 0.7, 0.85, weights_of=0)], 211, 13, 29, mult=0.6),
+    # five layers of three kinds: keys of 48 under values of 96 and of 64 under 128 (padded onto the matrix cores in
+    # bfloat16), four query heads a key head, a recurrence with keys of 80 (no power of two) and five taps, sixteen
+    # experts in eight groups, three a token; a width that is no power of two
+    "many": _case(300, 192, [_layer(*_MA, _moe(40, 16, 3, (8, 3)), 0.8, 1.2), _layer(*_MB, _dense(200), 1.0, 0.4),
+                             _layer(*_MA, _moe(40, 16, 3, (8, 3)), 0.8, 1.2, weights_of=0), _layer(*_MB, _dense(200), 1.0, 0.4, weights_of=1),
+                             _layer(_left(2, 1, 64, 128, 4, rot_dims=16, base=777.0, scaling=(2.0, 64, 4.0, 0.5)),
+                                    _right(2, 2, 32, 32, 3, 4, 4), None, 0.5, 0.5)], 997, 101, 13, mult=0.3),
 }
 
 
@@ -176,7 +186,8 @@ def tokens(name: str, n: int, seed: int) -> List[int]:
 #: request lengths per case: one token, a few, around pages' edges, long
 LENGTHS = {"pair": {"p0": 1, "p1": 6, "p2": 23, "p3": 49, "p4": 33, "p5": 16},
            "solo": {"s0": 2, "s1": 31, "s2": 17, "s3": 1, "s4": 40},
-           "wide": {"w0": 5, "w1": 70, "w2": 33, "w3": 129, "w4": 48}}
+           "wide": {"w0": 5, "w1": 70, "w2": 33, "w3": 129, "w4": 48},
+           "many": {"n0": 1, "n1": 37, "n2": 150, "n3": 64}}
 
 
 def requests(name: str) -> Dict[str, List[int]]:

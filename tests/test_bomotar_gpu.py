@@ -340,14 +340,14 @@ def _ref(name, rid, dtype):
     return _REFS[key]
 
 
-@pytest.mark.parametrize("name", ["pair", "solo", "wide"])
+@pytest.mark.parametrize("name", ["pair", "solo", "wide", "many"])
 def test_each_part_alone_matches_its_plain_function(dirs, name):
     import bomotar_mechanisms
     bomotar_mechanisms.check(dirs[name], name, DEV, 2e-5)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["pair", "solo", "wide"])
+@pytest.mark.parametrize("name", ["pair", "solo", "wide", "many"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_every_cutting_matches_plain(dirs, name, mode, dtype):
     reqs = cases.requests(name)
